@@ -37,9 +37,58 @@ class RopeScaling:
 
 
 @dataclass(frozen=True)
+class LayerSpec:
+    """One layer of a model whose layers differ from each other (a hybrid stack): which token mixer it
+    has, the mixer's own sizes, and the width of its feed-forward sublayer (0: the layer has none).
+
+    ``attention``: softmax attention over a paged cache, `heads` query heads over `kv_heads` key / value
+    heads, queries and keys of `dim`, values of `vdim`; `window` (None: the whole context) keeps the
+    keys j with 0 <= i - j < window; `sink` adds one to the softmax's denominator (a key of score 0 and no
+    value); `scale` multiplies the scores; `rope` says whether positions rotate q and k; `v_mix`: the
+    layer's values are blended with those of the first such layer of the stack, by a learned scalar.
+    ``delta``: a gated delta-rule recurrence per head over a [dim, vdim] state, q / k shared by
+    `heads // kv_heads` heads, each of q, k, v behind a causal convolution of `conv` taps."""
+    kind: str                       # "attention" | "delta"
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    ff: int = 0
+    window: Optional[int] = None
+    scale: float = 1.0
+    sink: bool = False
+    rope: bool = False
+    v_mix: bool = False
+    conv: int = 0
+
+    @property
+    def group(self) -> int:
+        return self.heads // self.kv_heads
+
+    @property
+    def qk_heads(self) -> int:
+        """Heads of the q projection: every query head for attention, the shared q / k heads for the delta rule."""
+        return self.heads if self.kind == "attention" else self.kv_heads
+
+    @property
+    def v_heads(self) -> int:
+        return self.kv_heads if self.kind == "attention" else self.heads
+
+    def mixer_param_count(self, width: int) -> int:
+        qn, kn, vn = self.qk_heads * self.dim, self.kv_heads * self.dim, self.v_heads * self.vdim
+        n = width * (qn + kn + vn) + self.heads * self.vdim * width
+        if self.kind == "attention":
+            return n + qn + kn + vn + 1
+        return n + self.conv * (qn + kn + vn) + 2 * self.heads * width + 2 * self.heads + self.vdim + self.heads * self.vdim * width
+
+    def ff_param_count(self, width: int) -> int:
+        return 3 * width * self.ff + 2 * self.ff + width if self.ff else 0
+
+
+@dataclass(frozen=True)
 class ModelSpec:
     name: str
-    family: str                     # "llama" | "gpt2"
+    family: str                     # "llama" | "gpt2" | "letarax"
     num_layers: int
     hidden_size: int
     num_heads: int
@@ -64,6 +113,19 @@ class ModelSpec:
     qkv_bias: bool = False
     o_bias: bool = False
     sliding_window: Optional[int] = None
+    # hybrid stacks (family "letarax"): one entry per layer; the scalar fields above then hold the width, the
+    # vocabulary and, for the sizes that differ per layer, the largest value over the layers
+    layer_specs: tuple = ()
+
+    @property
+    def is_hybrid(self) -> bool:
+        return bool(self.layer_specs)
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        """Some layer keeps a per-sequence state that lives in the sequence's slot (not in cache blocks): a sequence
+        cannot change slots without its state being moved along."""
+        return any(l.kind == "delta" for l in self.layer_specs)
 
     def check_context(self, max_seq_len: int):
         """Attention here is over the whole context. A checkpoint trained with a sliding window gives
@@ -99,6 +161,8 @@ class ModelSpec:
 
     def layer_param_count(self) -> int:
         h, i = self.hidden_size, self.intermediate_size
+        if self.is_hybrid:      # (the mean: the partitioner weighs layers equally)
+            return sum(l.mixer_param_count(h) + l.ff_param_count(h) + (4 if l.ff else 2) * h for l in self.layer_specs) // len(self.layer_specs)
         if self.is_llama:
             return h * self.qkv_size + self.q_size * h + 3 * h * i + 2 * h + self._attn_bias_count()
         # GPT-2: c_attn, c_proj, c_fc, mlp c_proj, all with biases, two LayerNorms
@@ -138,12 +202,62 @@ class ModelSpec:
         d = asdict(self)
         return d
 
+    @staticmethod
+    def from_letarax_config(cfg: Dict[str, Any], name: str = "") -> "ModelSpec":
+        """Letarax: a hybrid stack described layer by layer. ``layers`` lists for each layer its ``type``
+        (``attention``: windowed softmax attention with a sink and no rotation, ``delta``: gated delta rule),
+        the mixer's sizes (``mixer``: heads, kv_heads, dim, vdim; attention: mask.size, scale, v_mix;
+        delta: conv) and its feed-forward (``mlp``: kind ``dense`` with ``ff``, or null). ``width``,
+        ``vocab`` and ``norm.eps`` are the model's own. The output head is the embedding table."""
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m, mlp = l["mixer"], l.get("mlp")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported (dense is)")
+            ff = int(mlp["ff"]) if mlp is not None else 0
+            if int(m["heads"]) % int(m["kv_heads"]):
+                raise ValueError(f"layer {i}: {m['heads']} heads over {m['kv_heads']} key / value heads")
+            common = dict(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), ff=ff)
+            if l["type"] == "attention":
+                win = (m.get("mask") or {}).get("size")
+                layers.append(LayerSpec("attention", **common, window=int(win) if win else None,
+                                        scale=float(m.get("scale", float(m["dim"]) ** -0.5)), sink=True, rope=False,
+                                        v_mix=bool(m.get("v_mix", False))))
+            elif l["type"] == "delta":
+                layers.append(LayerSpec("delta", **common, conv=int(m["conv"]), scale=float(m["dim"]) ** -0.5))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        if not layers:
+            raise ValueError("a model needs at least one layer")
+        return ModelSpec(
+            name=name or "letarax", family="letarax", num_layers=len(layers), hidden_size=int(cfg["width"]),
+            num_heads=max(l.heads for l in layers), num_kv_heads=max(l.kv_heads for l in layers),
+            head_dim=max(max(l.dim, l.vdim) for l in layers), intermediate_size=max(l.ff for l in layers),
+            vocab_size=int(cfg["vocab"]), max_position=1 << 30, norm_eps=float(cfg["norm"]["eps"]),
+            tie_embeddings=True, bos_token_id=cfg.get("bos_token_id"), eos_token_id=_scalar_eos(cfg.get("eos_token_id")),
+            hf_type="letarax", layer_specs=tuple(layers))
+
+    def letarax_config(self) -> Dict[str, Any]:
+        """The inverse of `from_letarax_config`."""
+        out = []
+        for l in self.layer_specs:
+            if l.kind == "attention":
+                m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                     "mask": {"size": l.window}, "v_mix": l.v_mix}
+            else:
+                m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "conv": l.conv}
+            out.append({"type": l.kind, "mixer": m, "mlp": {"kind": "dense", "ff": l.ff} if l.ff else None})
+        return {"architecture": "Letarax", "layers": out, "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size,
+                "width": self.hidden_size, "bos_token_id": self.bos_token_id, "eos_token_id": self.eos_token_id}
+
     # ---- constructors ------------------------------------------------------
     @staticmethod
     def from_hf_config(cfg: Dict[str, Any], name: str = "") -> "ModelSpec":
         """Build a spec from the dict form of a Hugging Face ``config.json``."""
         mt = cfg.get("model_type", "")
         archs = cfg.get("architectures") or []
+        if cfg.get("architecture") == "Letarax":
+            return ModelSpec.from_letarax_config(cfg, name=name)
         if mt == "gpt2" or any("GPT2" in a for a in archs):
             if cfg.get("activation_function", "gelu_new") != "gelu_new" or cfg.get("scale_attn_by_inverse_layer_idx"):
                 raise ValueError("GPT-2 variants other than gelu_new MLPs with plain 1/sqrt(d) attention scaling are not supported")
@@ -274,6 +388,8 @@ class ModelSpec:
 
     def hf_config(self) -> Dict[str, Any]:
         """The inverse of `from_hf_config`: a config.json dict for this spec."""
+        if self.is_hybrid:
+            return self.letarax_config()
         if self.is_gpt2:
             return {
                 "model_type": "gpt2", "architectures": ["GPT2LMHeadModel"],

@@ -13,6 +13,19 @@ Logical layout (all matrices `[out_features, in_features]`, i.e. what ``nn.Linea
   final_norm_w (+final_norm_b)   [H]     last stage
   lm_head      [V, H]            last stage (aliases `embed` data when tied)
 
+Hybrid stacks (`spec.layer_specs`, the Letarax checkpoint names ``embed``, ``l{i}.norm1`` / ``norm1b`` /
+``norm2`` / ``norm2b``, ``l{i}.mix.*``, ``l{i}.mlp.*``, ``final.norm``) use per layer:
+
+               ln1_w, ln1b_w     [H]     norm before / after the mixer (stored as the distance from one)
+  attention:   w_qkv, b_qkv      [Hq*d + G*d + G*dv, H]  q, k, v concatenated
+               vmix              []      blend weight of the value mixing
+  delta:       w_in              [G*d + G*d + Hv*dv + Hv*dv + Hv + Hv, H]   q, k, v, output gate, beta, decay
+               conv_w            [G*d + G*d + Hv*dv, taps]                    causal convolutions of q, k, v
+               A_log, dt_bias    [Hv]    o_norm_w [dv]
+               w_o               [H, heads*dv]
+  feed-forward ln2_w, ln2b_w, w_gate, b_gate, w_up, b_up [I, H] / [I], w_down, b_down
+  lm_head = embed.
+
 A stage materialises only what its `StagePlan` owns.  The reference instead loads the full
 model in every process (orchestration.py:39-47, Worker1.py:60-75).
 
@@ -103,9 +116,102 @@ def _randn(name, shape, seed, device, dtype, std=0.02):
     return t.to(dtype)
 
 
+def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
+    """Random weights of a hybrid stack, scaled so that activations stay of order one through any depth
+    (projections at 1 / sqrt(fan-in), embedding at one) and every bias, convolution tap and gate matters."""
+    H, V = spec.hidden_size, spec.vocab_size
+    w = StageWeights(spec, plan)
+    rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
+    if plan.has_embed or plan.has_head:
+        w.embed = rn("embed", (V, H), 1.0)
+    for i in plan.layers:
+        ls, p = spec.layer_specs[i], f"layers.{i}."
+        qn, kn, vn, on = ls.qk_heads * ls.dim, ls.kv_heads * ls.dim, ls.v_heads * ls.vdim, ls.heads * ls.vdim
+        l: Dict[str, torch.Tensor] = {"ln1_w": rn(p + "ln1_w", (H,), 0.1), "ln1b_w": rn(p + "ln1b_w", (H,), 0.1)}
+        if ls.kind == "attention":
+            l["w_qkv"] = rn(p + "w_qkv", (qn + kn + vn, H), H ** -0.5)
+            l["b_qkv"] = rn(p + "b_qkv", (qn + kn + vn,), 0.3)
+            l["vmix"] = torch.full((), 0.25 + 0.5 * ((i * 7919 + seed) % 10) / 10.0, device=device, dtype=dtype)
+        else:
+            l["w_in"] = rn(p + "w_in", (qn + kn + vn + on + 2 * ls.heads, H), H ** -0.5)
+            l["conv_w"] = rn(p + "conv_w", (qn + kn + vn, ls.conv), 0.6)
+            l["A_log"] = rn(p + "A_log", (ls.heads,), 0.5)
+            l["dt_bias"] = rn(p + "dt_bias", (ls.heads,), 0.5)
+            l["o_norm_w"] = torch.ones(ls.vdim, device=device, dtype=dtype) + rn(p + "o_norm_w", (ls.vdim,), 0.1)
+        l["w_o"] = rn(p + "w_o", (H, on), on ** -0.5)
+        if ls.ff:
+            l["ln2_w"], l["ln2b_w"] = rn(p + "ln2_w", (H,), 0.1), rn(p + "ln2b_w", (H,), 0.1)
+            l["w_gate"], l["b_gate"] = rn(p + "w_gate", (ls.ff, H), H ** -0.5), rn(p + "b_gate", (ls.ff,), 0.2)
+            l["w_up"], l["b_up"] = rn(p + "w_up", (ls.ff, H), H ** -0.5), rn(p + "b_up", (ls.ff,), 0.2)
+            l["w_down"], l["b_down"] = rn(p + "w_down", (H, ls.ff), ls.ff ** -0.5), rn(p + "b_down", (H,), 0.2)
+        w.layers.append(l)
+    if plan.has_head:
+        w.final_norm_w = rn("final_norm_w", (H,), 0.1)
+        w.lm_head = w.embed
+    return w
+
+
+def _load_hybrid_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
+    w = StageWeights(spec, plan)
+    get = lambda name: rd.get(name).to(device=device, dtype=dtype)
+    if plan.has_embed or plan.has_head:
+        w.embed = get("embed")
+    for i in plan.layers:
+        ls, p = spec.layer_specs[i], f"l{i}."
+        m = p + "mix."
+        l = {"ln1_w": get(p + "norm1"), "ln1b_w": get(p + "norm1b"), "w_o": get(m + "o")}
+        if ls.kind == "attention":
+            l["w_qkv"] = torch.cat([get(m + x) for x in "qkv"], dim=0)
+            l["b_qkv"] = torch.cat([get(m + x + ".b") for x in "qkv"], dim=0)
+            l["vmix"] = get(m + "vmix").reshape(())
+        else:
+            l["w_in"] = torch.cat([get(m + x) for x in ("q", "k", "v", "g", "b", "a")], dim=0)
+            l["conv_w"] = torch.cat([get(m + x + ".conv") for x in "qkv"], dim=0)
+            l["A_log"], l["dt_bias"], l["o_norm_w"] = get(m + "A_log"), get(m + "dt_bias"), get(m + "norm")
+        if ls.ff:
+            f = p + "mlp."
+            l.update({"ln2_w": get(p + "norm2"), "ln2b_w": get(p + "norm2b"),
+                      "w_gate": get(f + "gate"), "b_gate": get(f + "gate.b"), "w_up": get(f + "up"), "b_up": get(f + "up.b"),
+                      "w_down": get(f + "down"), "b_down": get(f + "down.b")})
+        w.layers.append(l)
+    if plan.has_head:
+        w.final_norm_w = get("final.norm")
+        w.lm_head = w.embed
+    return w
+
+
+def export_letarax_state_dict(w: StageWeights) -> Dict[str, torch.Tensor]:
+    """Logical -> checkpoint names for a hybrid stack held by one stage (tests, `save` of random models)."""
+    spec, sd = w.spec, {"embed": w.embed, "final.norm": w.final_norm_w}
+    for i, l in zip(w.plan.layers, w.layers):
+        ls, p = spec.layer_specs[i], f"l{i}."
+        m = p + "mix."
+        qn, kn, vn, on = ls.qk_heads * ls.dim, ls.kv_heads * ls.dim, ls.v_heads * ls.vdim, ls.heads * ls.vdim
+        sd[p + "norm1"], sd[p + "norm1b"], sd[m + "o"] = l["ln1_w"], l["ln1b_w"], l["w_o"]
+        if ls.kind == "attention":
+            for x, t, b in zip("qkv", torch.split(l["w_qkv"], [qn, kn, vn]), torch.split(l["b_qkv"], [qn, kn, vn])):
+                sd[m + x], sd[m + x + ".b"] = t, b
+            sd[m + "vmix"] = l["vmix"]
+        else:
+            parts = torch.split(l["w_in"], [qn, kn, vn, on, ls.heads, ls.heads])
+            for x, t in zip(("q", "k", "v", "g", "b", "a"), parts):
+                sd[m + x] = t
+            for x, t in zip("qkv", torch.split(l["conv_w"], [qn, kn, vn])):
+                sd[m + x + ".conv"] = t
+            sd[m + "A_log"], sd[m + "dt_bias"], sd[m + "norm"] = l["A_log"], l["dt_bias"], l["o_norm_w"]
+        if ls.ff:
+            f = p + "mlp."
+            sd[p + "norm2"], sd[p + "norm2b"] = l["ln2_w"], l["ln2b_w"]
+            for x in ("gate", "up", "down"):
+                sd[f + x], sd[f + x + ".b"] = l["w_" + x], l["b_" + x]
+    return {k: v.detach().clone().contiguous() for k, v in sd.items()}
+
+
 def random_stage_weights(spec: ModelSpec, plan: StagePlan, seed: int = 0, device="cpu",
                          dtype=torch.float32) -> StageWeights:
     """Random-init weights of the given architecture for one stage."""
+    if spec.is_hybrid:
+        return _random_hybrid_weights(spec, plan, seed, device, dtype)
     H, I, V = spec.hidden_size, spec.intermediate_size, spec.vocab_size
     w = StageWeights(spec, plan)
     need_embed = plan.has_embed or (plan.has_head and spec.tie_embeddings)
@@ -195,6 +301,11 @@ def load_stage_weights(model_dir: str, spec: ModelSpec, plan: StagePlan, device=
                        dtype=torch.float32, reader: Optional[CheckpointReader] = None) -> StageWeights:
     """Read exactly this stage's tensors from a HF checkpoint directory."""
     rd = reader or CheckpointReader(model_dir)
+    if spec.is_hybrid:
+        w = _load_hybrid_weights(rd, spec, plan, device, dtype)
+        if reader is None:
+            rd.close()
+        return w
     w = StageWeights(spec, plan)
 
     def get(name):

@@ -180,7 +180,7 @@ class StageRuntime:
         Anything else — a prefill chunk, also one made only of 1-token prompts — runs eagerly and
         leaves the micro-batch's captured state alone."""
         ex = self.ex
-        return (desc.is_decode and hasattr(ex, "decode_step") and not self.debug_top5
+        return (desc.is_decode and hasattr(ex, "decode_step") and not self.debug_top5 and desc.score_rows is None
                 and desc.num_seqs in getattr(ex, "graph_sizes", (desc.num_seqs,)))
 
     def result_count(self, desc: StepBatch) -> int:
@@ -317,7 +317,9 @@ class StageRuntime:
             out = self.ex.decode_step(desc, x)
         else:
             out = self.ex.forward(desc, x)
-            if L.is_last:
+            if L.is_last and desc.score_rows is not None:
+                pass                  # a scoring step: the logits of the rows it names are its result, nothing is sampled
+            elif L.is_last:
                 if self.debug_top5:
                     self._log_top5(desc, out)
                 out = self.ex.sample(desc, out)
@@ -331,7 +333,9 @@ class StageRuntime:
 
         # ---- output ----------------------------------------------------------------------
         result = None
-        if L.is_last:
+        if L.is_last and desc.score_rows is not None:
+            result = out              # (no token comes of it, so nothing is fed back to stage 0)
+        elif L.is_last:
             result = out
             if L.num_stages == 1:
                 self._local_fb[mb] = out

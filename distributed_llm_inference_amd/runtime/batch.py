@@ -29,7 +29,7 @@ KIND_BARRIER = 5     # drain all outstanding work, then meet every other stage a
 
 _MAGIC = 0x444C4942  # "DLIB"
 _HEAD = "<IiiiiiiIii"   # magic, kind, step id, micro-batch, B, tokens (-1: none), table ints, flags, growth entries, live rows
-_F_REPLAY, _F_COMPACT = 1, 2
+_F_REPLAY, _F_COMPACT, _F_SCORE = 1, 2, 4
 
 
 @dataclass
@@ -66,6 +66,10 @@ class StepBatch:
     # packing per stage and step). `rows` = sequences of the micro-batch, `live` = those that decode.
     rows: int = -1
     live: int = -1
+    # Scoring step: the last stage returns the logits of these token rows (indices into the step's ragged
+    # token list, any position of a prompt chunk) and samples nothing. What a prompt's per-token scores
+    # and a replayed trace are made of.
+    score_rows: Optional[List[int]] = None
 
     @property
     def compact(self) -> bool:
@@ -114,6 +118,8 @@ class StepBatch:
             raise ValueError("table_slots / table_blocks mismatch")
         if not (len(self.grow_slots) == len(self.grow_pos) == len(self.grow_blocks)):
             raise ValueError("grow_slots / grow_pos / grow_blocks mismatch")
+        if self.score_rows is not None and any(not 0 <= r < self.num_tokens for r in self.score_rows):
+            raise ValueError("score_rows must index the step's tokens")
 
     # ---- wire format ------------------------------------------------------------------
     def to_bytes(self) -> bytes:
@@ -128,14 +134,16 @@ class StepBatch:
         for s, blocks in zip(self.table_slots, self.table_blocks):
             tb_flat += [s, len(blocks)] + list(blocks)
         ng = len(self.grow_slots)
+        flags = (_F_REPLAY if self.replay else 0) | (_F_SCORE if self.score_rows is not None else 0)
         head = struct.pack(_HEAD, _MAGIC, self.kind, self.step_id, self.micro_batch, B, ntok,
-                           len(tb_flat), _F_REPLAY if self.replay else 0, ng, -1)
+                           len(tb_flat), flags, ng, -1)
         ints = np.asarray(self.slots + self.q_lens + self.ctx_lens + self.sample + self.top_k +
                           self.sample_steps + tb_flat + self.grow_slots + self.grow_pos + self.grow_blocks +
                           (self.token_ids or []), dtype="<i4")
         flts = np.asarray(self.temperature + self.top_p, dtype="<f4")
         seeds = np.asarray(self.seeds, dtype="<i8")
-        return head + ints.tobytes() + flts.tobytes() + seeds.tobytes()
+        tail = b"" if self.score_rows is None else np.asarray([len(self.score_rows)] + list(self.score_rows), dtype="<i4").tobytes()
+        return head + ints.tobytes() + flts.tobytes() + seeds.tobytes() + tail
 
     @staticmethod
     def from_bytes(buf: bytes) -> "StepBatch":
@@ -154,6 +162,11 @@ class StepBatch:
         flts = np.frombuffer(buf, dtype="<f4", count=2 * B, offset=off).tolist()
         off += 8 * B
         seeds = np.frombuffer(buf, dtype="<i8", count=B, offset=off).tolist()
+        off += 8 * B
+        score = None
+        if flags & _F_SCORE:
+            n = int(np.frombuffer(buf, dtype="<i4", count=1, offset=off)[0])
+            score = np.frombuffer(buf, dtype="<i4", count=n, offset=off + 4).tolist()
         f = [ints[i * B:(i + 1) * B] for i in range(6)]
         tb = ints[6 * B:6 * B + ntb]
         table_slots, table_blocks, i = [], [], 0
@@ -168,7 +181,7 @@ class StepBatch:
         return StepBatch(kind=kind, step_id=step_id, micro_batch=mb, slots=f[0], q_lens=f[1], ctx_lens=f[2],
                          sample=f[3], top_k=f[4], sample_steps=f[5], temperature=flts[:B], top_p=flts[B:],
                          seeds=seeds, table_slots=table_slots, table_blocks=table_blocks, token_ids=toks,
-                         replay=bool(replay), grow_slots=grow[0], grow_pos=grow[1], grow_blocks=grow[2])
+                         replay=bool(replay), grow_slots=grow[0], grow_pos=grow[1], grow_blocks=grow[2], score_rows=score)
 
 
 def control(kind: int, slots: Optional[List[int]] = None, step_id: int = 0) -> StepBatch:

@@ -515,6 +515,8 @@ class Engine:
         sizes = self._graph_sizes
         if len(sizes) < 2:
             return
+        if getattr(self.spec, "has_recurrent_state", False):
+            return                                   # a recurrent layer's state lives in the slot: rows stay where they are
         live = [r for r in mb.rows if r is not None]
         n = len(live)
         if n == 0 or n == len(mb.rows):
