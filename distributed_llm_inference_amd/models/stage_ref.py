@@ -38,7 +38,10 @@ class RefStage:
         spec.check_context(self.max_seq_len)
         if spec.is_llama:
             self.cos, self.sin = build_rope_table(spec, self.max_seq_len, self.device)
-        # slot -> per-layer [K, V] tensors of shape [len, Hkv, D]
+        if spec.is_hybrid and not (plan.has_embed and plan.has_head):
+            raise ValueError("a hybrid stack runs on one stage (its value mixing spans layers)")
+        # slot -> per-layer [K, V] tensors of shape [len, Hkv, D]; a delta-rule layer of a hybrid stack keeps
+        # [last conv inputs [taps-1, C], state [H, d, dv]] there instead
         self.cache: Dict[int, List[List[torch.Tensor]]] = {}
 
     # -- helpers --------------------------------------------------------------------------
@@ -50,10 +53,22 @@ class RefStage:
     def _slot_cache(self, slot: int):
         c = self.cache.get(slot)
         if c is None:
-            z = lambda: torch.zeros(0, self.spec.num_kv_heads, self.spec.head_dim, dtype=self.dtype, device=self.device)
-            c = [[z(), z()] for _ in self.plan.layers]
+            if self.spec.is_hybrid:
+                c = [self._fresh_layer_state(self.spec.layer_specs[i]) for i in self.plan.layers]
+            else:
+                z = lambda: torch.zeros(0, self.spec.num_kv_heads, self.spec.head_dim, dtype=self.dtype, device=self.device)
+                c = [[z(), z()] for _ in self.plan.layers]
             self.cache[slot] = c
         return c
+
+    def _fresh_layer_state(self, ls):
+        dev = self.device
+        if ls.kind == "attention":
+            return [torch.zeros(0, ls.kv_heads, ls.dim, dtype=self.dtype, device=dev),
+                    torch.zeros(0, ls.kv_heads, ls.vdim, dtype=self.dtype, device=dev)]
+        C = 2 * ls.kv_heads * ls.dim + ls.heads * ls.vdim
+        return [torch.zeros(ls.conv - 1, C, dtype=torch.float32, device=dev),
+                torch.zeros(ls.heads, ls.dim, ls.vdim, dtype=torch.float32, device=dev)]
 
     def release(self, slots: List[int]):
         for s in slots:
@@ -74,9 +89,102 @@ class RefStage:
         return R.gemm(hn, self.w.lm_head).float()
 
     # -- forward --------------------------------------------------------------------------
+    # -- hybrid stacks: fp32 residual stream, a norm on both sides of every sublayer ------------------------------
+    def _hybrid_layers(self, batch: StepBatch, h: torch.Tensor) -> torch.Tensor:
+        """h [T, width] fp32 -> the residual stream after this stage's layers. Matrix products take their
+        inputs in the compute dtype and accumulate in fp32; norms, scores, softmax, gates, decays and the
+        recurrent state are fp32 whatever the dtype."""
+        spec, dt, eps = self.spec, self.dtype, self.spec.norm_eps
+        T = h.shape[0]
+        lin = lambda x, w, b=None: R.gemm(x.to(dt), w, b, None, 1 if b is not None else 0)
+        for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+            if qlen > 0 and ctx == 0:
+                self.cache.pop(slot, None)            # a sequence's first tokens: whatever the slot held before is void
+        v_first = None
+        for li, l in enumerate(self.w.layers):
+            ls = spec.layer_specs[self.plan.layers[li]]
+            xn = R.rmsnorm(h, l["ln1_w"], eps, unit_offset=True)
+            H, G, d, dv = ls.heads, ls.kv_heads, ls.dim, ls.vdim
+            mixed = torch.empty(T, H * dv, dtype=torch.float32, device=self.device)
+            if ls.kind == "attention":
+                qkv = lin(xn, l["w_qkv"], l["b_qkv"])
+                q = qkv[:, :H * d].reshape(T, H, d).to(dt)
+                k = qkv[:, H * d:(H + G) * d].reshape(T, G, d).to(dt)
+                v = qkv[:, (H + G) * d:].reshape(T, G, dv)
+                if ls.v_mix:
+                    if v_first is None:
+                        v_first = v
+                    else:
+                        lam = l["vmix"].float()
+                        v = (1.0 - lam) * v + lam * v_first
+                v = v.to(dt)
+                t0 = 0
+                for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+                    if qlen == 0:
+                        continue
+                    kv = self._slot_cache(slot)[li]
+                    assert kv[0].shape[0] >= ctx, f"slot {slot}: cache has {kv[0].shape[0]} tokens, step says {ctx}"
+                    kv[0] = torch.cat([kv[0][:ctx], k[t0:t0 + qlen]])
+                    kv[1] = torch.cat([kv[1][:ctx], v[t0:t0 + qlen]])
+                    o = R.attention(q[t0:t0 + qlen], kv[0], kv[1], ctx, ls.scale, window=ls.window or 0, sink=ls.sink)
+                    mixed[t0:t0 + qlen] = o.reshape(qlen, H * dv)
+                    t0 += qlen
+            else:
+                qn, vn = G * d, H * dv
+                z = lin(xn, l["w_in"])
+                conv_in, gate = z[:, :2 * qn + vn], z[:, 2 * qn + vn:2 * qn + 2 * vn]
+                beta = torch.sigmoid(z[:, 2 * qn + 2 * vn:2 * qn + 2 * vn + H])
+                decay = torch.exp(-torch.exp(l["A_log"].float()) * torch.nn.functional.softplus(z[:, 2 * qn + 2 * vn + H:] + l["dt_bias"].float()))
+                t0 = 0
+                for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+                    if qlen == 0:
+                        continue
+                    st = self._slot_cache(slot)[li]
+                    y, st[0] = R.short_conv(conv_in[t0:t0 + qlen].to(dt), st[0], l["conv_w"])
+                    y = torch.nn.functional.silu(y.to(dt).float())
+                    qq = R.l2_unit(y[:, :qn].reshape(qlen, G, d)) * (d ** -0.5)
+                    kk = R.l2_unit(y[:, qn:2 * qn].reshape(qlen, G, d))
+                    o, st[1] = R.gated_delta_rule(qq, kk, y[:, 2 * qn:].reshape(qlen, H, dv), beta[t0:t0 + qlen],
+                                                  decay[t0:t0 + qlen], st[1])
+                    o = R.rmsnorm(o, l["o_norm_w"], eps) * torch.nn.functional.silu(gate[t0:t0 + qlen].to(dt).float()).reshape(qlen, H, dv)
+                    mixed[t0:t0 + qlen] = o.reshape(qlen, H * dv)
+                    t0 += qlen
+            h = h + R.rmsnorm(lin(mixed, l["w_o"]), l["ln1b_w"], eps, unit_offset=True)
+            if ls.ff:
+                xn = R.rmsnorm(h, l["ln2_w"], eps, unit_offset=True)
+                act = R.gelu_tanh(lin(xn, l["w_gate"], l["b_gate"]).to(dt).float()) * lin(xn, l["w_up"], l["b_up"]).to(dt).float()
+                h = h + R.rmsnorm(lin(act, l["w_down"], l["b_down"]), l["ln2b_w"], eps, unit_offset=True)
+        return h
+
+    def _forward_hybrid(self, batch: StepBatch, x: torch.Tensor) -> torch.Tensor:
+        T = batch.num_tokens
+        ids = torch.as_tensor(x).to(self.device).long().reshape(-1)
+        assert ids.numel() == T, f"expected {T} token ids, got {ids.numel()}"
+        h = self._hybrid_layers(batch, self.w.embed[ids].float())
+        self.last_hidden = h
+        rows = self._out_rows(batch)
+        if not rows:
+            return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+        hn = R.rmsnorm(h[rows], self.w.final_norm_w, self.spec.norm_eps, unit_offset=True)
+        return R.gemm(hn.to(self.dtype), self.w.lm_head).float()
+
+    @staticmethod
+    def _out_rows(batch: StepBatch) -> List[int]:
+        """Token rows whose logits a step returns: the rows it asks scores for, else the last row of every sampled sequence."""
+        if batch.score_rows is not None:
+            return list(batch.score_rows)
+        rows, t0 = [], 0
+        for qlen, s in zip(batch.q_lens, batch.sample):
+            if s and qlen > 0:
+                rows.append(t0 + qlen - 1)
+            t0 += qlen
+        return rows
+
     @torch.no_grad()
     def forward(self, batch: StepBatch, x: torch.Tensor) -> torch.Tensor:
         spec = self.spec
+        if spec.is_hybrid:
+            return self._forward_hybrid(batch, x)
         T = batch.num_tokens
         positions = torch.tensor([c + i for c, q in zip(batch.ctx_lens, batch.q_lens) for i in range(q)],
                                  dtype=torch.long, device=self.device)
@@ -127,12 +235,8 @@ class RefStage:
                 h = R.gemm(act, l["w_down"], l["b_down"], h, 3).to(self.dtype)
         if not self.plan.has_head:
             return h
-        # last stage: only the final position of each sequence that asks for a token
-        rows, t0 = [], 0
-        for qlen, s in zip(batch.q_lens, batch.sample):
-            if s and qlen > 0:
-                rows.append(t0 + qlen - 1)
-            t0 += qlen
+        # last stage: only the final position of each sequence that asks for a token (or the rows to be scored)
+        rows = self._out_rows(batch)
         if not rows:
             return torch.empty(0, spec.vocab_size, dtype=torch.float32, device=self.device)
         hn = self._norm(h[rows], self.w.final_norm_w, self.w.final_norm_b)

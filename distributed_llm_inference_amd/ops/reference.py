@@ -7,9 +7,10 @@ import torch
 import torch.nn.functional as F
 
 
-def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, unit_offset: bool = False) -> torch.Tensor:
+    """`unit_offset`: the weight is stored as its distance from one (the scale is 1 + w)."""
     xf = x.float()
-    return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * (w.float() + 1.0 if unit_offset else w.float())
 
 
 def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> torch.Tensor:
@@ -46,9 +47,12 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch
     return torch.cat([a * c - b * s, b * c + a * s], dim=-1)
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, scale: float) -> torch.Tensor:
-    """One sequence. q [Tq, Hq, D] are the tokens at absolute positions q_pos0.., k/v
-    [Tk, Hkv, D] hold positions 0..Tk-1 (Tk >= q_pos0 + Tq). Causal, GQA. Returns [Tq, Hq, D] fp32."""
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, scale: float,
+              window: int = 0, sink: bool = False, k_pos0: int = 0) -> torch.Tensor:
+    """One sequence. q [Tq, Hq, D] are the tokens at absolute positions q_pos0.., k [Tk, Hkv, D] and
+    v [Tk, Hkv, Dv] hold positions k_pos0..k_pos0+Tk-1 (reaching at least the last query). Causal, GQA.
+    `window` > 0: a query at i sees the keys j with 0 <= i - j < window. `sink`: the softmax's
+    denominator has one more term, exp(0), that carries no value. Returns [Tq, Hq, Dv] fp32."""
     Tq, Hq, D = q.shape
     Tk, Hkv, _ = k.shape
     g = Hq // Hkv
@@ -56,7 +60,47 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, sc
     vf = v.float().repeat_interleave(g, dim=1)
     s = torch.einsum("qhd,khd->hqk", q.float(), kf) * scale
     qpos = torch.arange(Tq, device=q.device).view(-1, 1) + q_pos0
-    kpos = torch.arange(Tk, device=q.device).view(1, -1)
-    s = s.masked_fill((kpos > qpos).unsqueeze(0), float("-inf"))
-    p = torch.softmax(s, dim=-1)
+    kpos = torch.arange(Tk, device=q.device).view(1, -1) + k_pos0
+    hidden = kpos > qpos
+    if window and window > 0:
+        hidden = hidden | (qpos - kpos >= window)
+    s = s.masked_fill(hidden.unsqueeze(0), float("-inf"))
+    if sink:
+        s = torch.cat([s, s.new_zeros(Hq, Tq, 1)], dim=-1)
+        p = torch.softmax(s, dim=-1)[..., :-1]
+    else:
+        p = torch.softmax(s, dim=-1)
     return torch.einsum("hqk,khd->qhd", p, vf)
+
+
+def short_conv(x: torch.Tensor, prev: torch.Tensor, taps: torch.Tensor):
+    """Causal per-channel convolution over time. x [T, C] new inputs, prev [K-1, C] the inputs before them
+    (zeros at a sequence's start), taps [C, K] with the last column on the current token. Returns
+    (y [T, C] fp32, the last K-1 inputs)."""
+    K = taps.shape[1]
+    full = torch.cat([prev.float(), x.float()], dim=0)
+    T = x.shape[0]
+    y = sum(full[j:j + T] * taps[:, j].float() for j in range(K))
+    return y, full[full.shape[0] - (K - 1):]
+
+
+def l2_unit(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    xf = x.float()
+    return xf * torch.rsqrt(xf.pow(2).sum(-1, keepdim=True) + eps)
+
+
+def gated_delta_rule(q, k, v, beta, decay, S):
+    """Token-by-token gated delta rule. q, k [T, G, d], v [T, H, dv], beta, decay [T, H], S [H, d, dv] fp32
+    (head h reads q / k head h // (H / G)). Per token: S <- decay S; u = beta (v - S^T k); S <- S + k u^T;
+    o = S^T q. Returns (o [T, H, dv], S)."""
+    T, H, _ = v.shape
+    g = H // q.shape[1]
+    qf, kf = q.float().repeat_interleave(g, dim=1), k.float().repeat_interleave(g, dim=1)
+    vf, S = v.float(), S.float().clone()
+    out = torch.empty(T, H, v.shape[2], dtype=torch.float32, device=v.device)
+    for t in range(T):
+        S = S * decay[t].float().view(H, 1, 1)
+        u = beta[t].float().view(H, 1) * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
+        S = S + kf[t].unsqueeze(2) * u.unsqueeze(1)
+        out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+    return out, S
