@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 ARCH = "gfx950"
 HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-fno-math-errno", "-fno-gpu-rdc",
-             "-Wno-unused-result"]
+             "-Wno-unused-result", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # kernels with hand-counted vmcnt waits: {source: kernel-name regex}; their ISA is linted after compiling
 LINTED = {"gemm_skinny.hip": "gemm_skinny_kernel", "gemm_a8w8.hip": "gemm_a8w8_kernel"}
 
@@ -49,7 +49,8 @@ def _lint(hipcc, src, regex):
                            f"first: {bad[0][0]}: {bad[0][1]}")
 
 
-def build(verbose: bool = True, force: bool = False) -> str:
+def build(verbose: bool = True, force: bool = False, comm: bool = True) -> str:
+    """`comm=False` leaves the communication library out (a single-stage run never loads it)."""
     import torch
     from torch.utils import cpp_extension as ce
 
@@ -92,7 +93,8 @@ def build(verbose: bool = True, force: bool = False) -> str:
         if verbose:
             print(f"[dlia.build] linked {out}", flush=True)
     build_runtime(verbose=verbose, force=force)
-    build_comm(verbose=verbose, force=force)
+    if comm:
+        build_comm(verbose=verbose, force=force)
     return out
 
 

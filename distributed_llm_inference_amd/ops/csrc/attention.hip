@@ -54,6 +54,10 @@ struct AttnParams {
   int max_blocks, num_blocks, qtiles, splits;
   float scale_log2;               // softmax scale * log2(e)
   int xcd_map;                    // prefill kernel: 0 plain order, 1 group i on XCD i % 8, r > 1: r XCDs per group (see there)
+  // Windowed instantiations (WIN): a query at position i sees the keys j with 0 <= i - j < window (0: the whole
+  // context); sink: the softmax's denominator has one more term exp(0) that carries no value (added once, where
+  // the row is normalised, so split and merged partials stay plain).
+  int window, sink;
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -61,7 +65,7 @@ constexpr float kNegInf = -__builtin_inff();
 // NW = waves per work item: 4 interleave the item's KV blocks and merge at the end (few items, long
 // contexts); 1 walks all of them alone with no LDS and no barrier (decode over thousands of
 // (sequence, kv head) items, where a 160-token context is 5 blocks and 4 waves would take 2, 1, 1, 1).
-template <int D, int NT, bool KV8, int NW, bool PF>
+template <int D, int NT, bool KV8, int NW, bool PF, bool WIN = false>
 __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) {
   constexpr int KS = D / 32;      // MFMA k-steps over the head dim (QK^T)
   constexpr int DT = D / 16;      // 16-row tiles of the head dim (PV)
@@ -107,8 +111,10 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
   const int tile_q_end = min(q_len, qp0 + QT);
   const int kv_len = tile_live ? min(ctx + tile_q_end, p.max_blocks * kBlockTokens) : 0;
   const int nb = (kv_len + kBlockTokens - 1) / kBlockTokens;
-  const int per = (nb + p.splits - 1) / p.splits;
-  const int kb0 = split * per, kb1 = min(nb, kb0 + per);
+  // windowed: blocks before the first key that the tile's first query still sees are never touched
+  const int kb_lo = (WIN && p.window > 0 && tile_live) ? max(0, ctx + qp0 - p.window + 1) / kBlockTokens : 0;
+  const int per = (max(nb - kb_lo, 0) + p.splits - 1) / p.splits;
+  const int kb0 = kb_lo + split * per, kb1 = min(nb, kb0 + per);
 
   // Q fragments (B operand): lane (c, quad) holds Q[c][s*32 + quad*8 .. +8]
   u32x4 qf[NT][KS];
@@ -206,7 +212,9 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int kpos = kb * kBlockTokens + kt * 16 + quad * 4 + r;
-          const float sc = kpos <= limit ? st[kt][nt][r] : kNegInf;
+          bool seen = kpos <= limit;
+          if constexpr (WIN) seen = seen && (p.window <= 0 || kpos + p.window > limit);
+          const float sc = seen ? st[kt][nt][r] : kNegInf;
           st[kt][nt][r] = sc;
           mx = fmaxf(mx, sc);
         }
@@ -275,6 +283,9 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
       lt += __shfl_xor(lt, 16, 64);
       lt += __shfl_xor(lt, 32, 64);
       if (col_qpos[nt] < 0) continue;
+      if constexpr (WIN) {
+        if (p.sink && p.splits == 1) lt += exp2f((0.f - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
+      }
       const float inv = lt > 0.f ? 1.f / lt : 0.f;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -325,6 +336,9 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
       lt += lw[w] * wgt[w];
     }
     if (col_qpos[nt] < 0) continue;
+    if constexpr (WIN) {
+      if (p.sink && p.splits == 1) lt += exp2f((0.f - m_safe) * p.scale_log2);
+    }
     const float inv = lt > 0.f ? 1.f / lt : 0.f;
     for (int dt = wave; dt < DT; dt += 4) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -344,14 +358,14 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
   }
 }
 
-template <int D, int NT, bool KV8>
-__global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) { paged_attn_body<D, NT, KV8, 4, true>(p, blockIdx.x); }
+template <int D, int NT, bool KV8, bool WIN = false>
+__global__ __launch_bounds__(256) void paged_attn_kernel(AttnParams p) { paged_attn_body<D, NT, KV8, 4, true, WIN>(p, blockIdx.x); }
 
 // One wave per item, one block in flight per wave, registers capped so that 3 waves share a SIMD:
 // latency is hidden by the other waves instead of by a second set of K/V registers.
-template <int D, bool KV8>
+template <int D, bool KV8, bool WIN = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 4))) void paged_attn_lean_kernel(AttnParams p) {
-  paged_attn_body<D, 1, KV8, 1, false>(p, blockIdx.x);
+  paged_attn_body<D, 1, KV8, 1, false, WIN>(p, blockIdx.x);
 }
 
 // The same one-wave-per-item body in a fixed number of 4-wave workgroups (one wave per SIMD) that walk the item list
@@ -396,6 +410,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
         acc += ov * wgt;
       }
     }
+    if (p.sink) lt += exp2f((0.f - (mt == kNegInf ? 0.f : mt)) * p.scale_log2);
     const float inv = lt > 0.f ? 1.f / lt : 0.f;
     const int head = kvh * p.g_real + (c & (g - 1));
     u32x2 v = {pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv)};
@@ -442,7 +457,7 @@ __device__ __forceinline__ float quad_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <int D, bool KV8>
+template <int D, bool KV8, bool WIN = false>
 __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
   constexpr int KS = D / 32, DT = D / 16, NT = 2, NC = 128;
   constexpr int BLOCK_BYTES = 2 * 2 * kBlockTokens * D;               // K slab + V slab of one head as bf16 (in LDS)
@@ -597,7 +612,9 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int kpos = kb * kBlockTokens + kt * 16 + quad * 4 + r;
-            const float sc = kpos <= limit ? st[kt][nt][r] : kNegInf;
+            bool seen = kpos <= limit;
+            if constexpr (WIN) seen = seen && (p.window <= 0 || kpos + p.window > limit);
+            const float sc = seen ? st[kt][nt][r] : kNegInf;
             st[kt][nt][r] = sc;
             mx = fmaxf(mx, sc);
           }
@@ -642,8 +659,10 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
   int tbl = 0;
   auto tbl_fill = [&](int kb) { tbl = (kb + lane < p.max_blocks) ? table[kb + lane] : 0; };
   auto tbl_at = [&](int kb) { return __builtin_amdgcn_readlane(tbl, kb & 63); };
-  tbl_fill(0);
-  if (nb > 0) { gload(tbl_at(0)); lstore(0); }
+  // windowed: the walk starts at the block of the first key that the tile's first query still sees
+  const int kb_lo = (WIN && p.window > 0 && tile_live) ? min(max(0, ctx + qp0 - p.window + 1) / kBlockTokens, nb) : 0;
+  tbl_fill(kb_lo & ~63);
+  if (nb > kb_lo) { gload(tbl_at(kb_lo)); lstore((kb_lo & 1) * BUF); }
   // Everything loaded so far (the Q fragments, block 0) has landed before the loop starts: vmcnt is
   // one in-order counter, so a wait for a prologue load placed inside the loop would also wait for
   // the prefetch of the next block that was issued just before it.
@@ -655,7 +674,13 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
   // happens to need none. With both forms in one loop the accumulators lived in different registers
   // in each and the compiler reconciled them with a dozen v_mov_b64 per block; VALU and MFMA time add
   // up in this kernel (66 % + 32 % of SIMD time), so those copies were not free.
-  const int nb_full = tile_live ? min(nb, (ctx + qp0 + 1) / kBlockTokens) : 0;      // workgroup-uniform
+  int nb_full = tile_live ? min(nb, (ctx + qp0 + 1) / kBlockTokens) : 0;      // workgroup-uniform
+  // windowed: blocks that start before the window of the tile's LAST query need the mask as well
+  int kb_mid = kb_lo;
+  if constexpr (WIN) {
+    nb_full = max(nb_full, kb_lo);
+    if (p.window > 0 && tile_live) kb_mid = min(nb_full, max(kb_lo, (max(0, ctx + tile_q_end - p.window) + kBlockTokens - 1) / kBlockTokens));
+  }
   auto run = [&](int kb_begin, int kb_end, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
     for (int kb = kb_begin; kb < kb_end; ++kb) {
@@ -670,13 +695,17 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
       __syncthreads();
     }
   };
-  run(0, nb_full, std::false_type{});
+  if constexpr (WIN) run(kb_lo, kb_mid, std::true_type{});
+  run(kb_mid, nb_full, std::false_type{});
   run(nb_full, nb, std::true_type{});
 
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const float lt = quad_sum(l[nt]);
+    float lt = quad_sum(l[nt]);
     if (col_qpos[nt] < 0) continue;
+    if constexpr (WIN) {
+      if (p.sink) lt += exp2f((0.f - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
+    }
     const float inv = lt > 0.f ? 1.f / lt : 0.f;
     int le = lane;
     asm volatile("" : "+v"(le));                   // recompute from the lane id instead of keeping the prologue's values live
@@ -695,7 +724,9 @@ template <int D>
 static void launch_prefill_attn(const AttnParams& p, hipStream_t stream) {
   const long nitems = p.xcd_map > 1 ? 8L * ((p.qtiles + p.xcd_map - 1) / p.xcd_map) : (long)p.B * p.Hkv * p.qtiles;
   constexpr size_t smem = 2 * (4 * kBlockTokens * D + 256);      // two bf16 blocks + their scales
+  const bool win = p.window > 0 || p.sink;
   if (p.kv_scale) hipLaunchKernelGGL((prefill_attn_kernel<D, true>), dim3((unsigned)nitems), dim3(256), smem, stream, p);
+  else if (win)   hipLaunchKernelGGL((prefill_attn_kernel<D, false, true>), dim3((unsigned)nitems), dim3(256), smem, stream, p);
   else            hipLaunchKernelGGL((prefill_attn_kernel<D, false>), dim3((unsigned)nitems), dim3(256), smem, stream, p);
 }
 
@@ -715,7 +746,12 @@ static void launch_attn(const AttnParams& p, hipStream_t stream) {
   const long thr = wave_per_item_threshold();
   const char* pe = getenv("DLIA_ATTN_PERSIST");               // read per launch (a captured graph keeps what it was captured with)
   const long persist = pe ? atol(pe) : 0L;
-  if (NT == 1 && thr > 0 && nitems >= thr && persist > 0 && nitems >= persist * 4 && !p.kv_scale) {
+  if ((p.window > 0 || p.sink) && !p.kv_scale) {             // windowed / sink instantiations (bf16 cache)
+    if (NT == 1 && thr > 0 && nitems >= thr)
+      hipLaunchKernelGGL((paged_attn_lean_kernel<D, false, true>), dim3((unsigned)nitems), dim3(64), 0, stream, p);
+    else
+      hipLaunchKernelGGL((paged_attn_kernel<D, NT, false, true>), dim3((unsigned)nitems), dim3(256), smem, stream, p);
+  } else if (NT == 1 && thr > 0 && nitems >= thr && persist > 0 && nitems >= persist * 4 && !p.kv_scale) {
     hipLaunchKernelGGL((paged_attn_lean_persist_kernel<D, false>), dim3((unsigned)persist), dim3(256), 0, stream, p, nitems);
   } else if (NT == 1 && thr > 0 && nitems >= thr) {
     if (p.kv_scale) hipLaunchKernelGGL((paged_attn_lean_kernel<D, true>), dim3((unsigned)nitems), dim3(64), 0, stream, p);
@@ -765,9 +801,10 @@ extern "C" void dlia_paged_attention(void* out, const void* qkv, const void* kv_
                                      const int* q_start, const int* ctx_lens, const int* block_table,
                                      const int* slots, float* partial, int B, int max_q_len, int Hq,
                                      int Hkv, int D, int table_rows, int max_blocks, int num_blocks,
-                                     long ldq, long ldo, float scale, int splits, hipStream_t stream) {
+                                     long ldq, long ldo, float scale, int splits, hipStream_t stream, int window, int sink) {
   if (B <= 0 || max_q_len <= 0) return;
   AttnParams p;
+  p.window = kv_scale ? 0 : window; p.sink = kv_scale ? 0 : sink;
   p.out = (bf16*)out; p.ldo = ldo; p.q = (const bf16*)qkv; p.ldq = ldq; p.kv = (const bf16*)kv_cache; p.kv_scale = kv_scale;
   p.q_start = q_start; p.ctx_lens = ctx_lens; p.block_table = block_table; p.slots = slots; p.table_rows = table_rows; p.partial = partial;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv;

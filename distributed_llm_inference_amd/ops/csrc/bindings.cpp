@@ -444,9 +444,10 @@ int64_t attention_ws_floats(int64_t B, int64_t max_q_len, int64_t Hq, int64_t Hk
 static void paged_attention_impl(Tensor out, const Tensor& qkv, const Tensor& kv_cache, OptTensor kv_scale,
                                  const Tensor& q_start, const Tensor& ctx_lens, const Tensor& block_table,
                                  OptTensor slots, OptTensor partial, int64_t max_q_len, int64_t Hq, int64_t Hkv,
-                                 int64_t D, double scale, int64_t splits) {
+                                 int64_t D, double scale, int64_t splits, int64_t window = 0, bool sink = false) {
   DLIA_ON_DEVICE_OF(out);
   check_bf16(out, "out"); check_bf16(qkv, "qkv"); check_rows(out, "out"); check_rows(qkv, "qkv");
+  DLIA_CHECK(window >= 0 && (!kv_scale.has_value() || (window == 0 && !sink)), "window / sink: bf16 cache only, window >= 0");
   DLIA_CHECK(D == 64 || D == 128, "head_dim must be 64 or 128");
   DLIA_CHECK(Hq % Hkv == 0, "Hq must be a multiple of Hkv");
   const int64_t g = Hq / Hkv;
@@ -481,7 +482,28 @@ static void paged_attention_impl(Tensor out, const Tensor& qkv, const Tensor& kv
                        kv_scale.has_value() ? kv_scale->data_ptr<float>() : nullptr, q_start.data_ptr<int>(),
                        ctx_lens.data_ptr<int>(), block_table.data_ptr<int>(), slp, pp, (int)B, (int)max_q_len, (int)Hq,
                        (int)Hkv, (int)D, (int)block_table.size(0), (int)block_table.size(1), (int)geo.num_blocks, qkv.stride(0),
-                       out.stride(0), (float)scale, sp, cur_stream());
+                       out.stride(0), (float)scale, sp, cur_stream(), (int)window, sink ? 1 : 0);
+}
+
+// Causal attention restricted to a sliding window (0: none), optionally with a softmax sink, over the bf16 cache.
+void paged_attention_window(Tensor out, const Tensor& qkv, const Tensor& kv_cache, const Tensor& q_start,
+                            const Tensor& ctx_lens, const Tensor& block_table, OptTensor slots, OptTensor partial,
+                            int64_t max_q_len, int64_t Hq, int64_t Hkv, int64_t D, double scale, int64_t splits,
+                            int64_t window, bool sink) {
+  paged_attention_impl(out, qkv, kv_cache, c10::nullopt, q_start, ctx_lens, block_table, slots, partial, max_q_len, Hq, Hkv, D,
+                       scale, splits, window, sink);
+}
+
+void value_mix(Tensor qkv, Tensor vfirst, OptTensor lam, int64_t mix, int64_t v_off, int64_t v_cols) {
+  DLIA_ON_DEVICE_OF(qkv);
+  check_bf16(qkv, "qkv"); check_f32(vfirst, "vfirst");
+  DLIA_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && v_off >= 0 && v_cols >= 0 && v_off + v_cols <= qkv.size(1), "value_mix: columns");
+  DLIA_CHECK(vfirst.numel() >= qkv.size(0) * v_cols && (mix == 1 || mix == 2), "value_mix: buffer / mode");
+  const float* lp = nullptr;
+  if (lam.has_value()) { check_f32(*lam, "lam"); DLIA_CHECK(lam->numel() >= 1, "lam"); lp = lam->data_ptr<float>(); }
+  DLIA_CHECK(mix != 2 || lp, "mix 2 needs lam");
+  dlia_value_mix(qkv.data_ptr(), vfirst.data_ptr<float>(), lp, (int)mix, (int)qkv.size(0), (int)v_off, (int)v_cols, qkv.stride(0),
+                 cur_stream());
 }
 
 void paged_attention(Tensor out, const Tensor& qkv, const Tensor& kv_cache, const Tensor& q_start,
@@ -628,9 +650,209 @@ void advance(Tensor x, int64_t delta) {
   dlia_advance_i32(x.data_ptr<int>(), (int)x.numel(), (int)delta, cur_stream());
 }
 
+
+// ---- fp32-residual models: any-shape GEMM, sandwich norms, windowed attention, delta rule ----------------------
+inline bool is_f32(const Tensor& t) { return t.scalar_type() == at::kFloat; }
+inline void check_act(const Tensor& t, const char* name) {
+  check_dev(t, name);
+  DLIA_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, name, " must be float32 or bfloat16");
+}
+inline void check_mat(const Tensor& t, const char* name) {
+  DLIA_CHECK(t.dim() == 2 && (t.size(1) == 1 || t.stride(1) == 1), name, " must be 2-D with unit inner stride");
+}
+inline const float* opt_f32(OptTensor t, int64_t n, const char* name) {
+  if (!t.has_value()) return nullptr;
+  check_f32(*t, name);
+  DLIA_CHECK(t->numel() >= n, name, " has too few elements");
+  return t->data_ptr<float>();
+}
+
+void embed32(Tensor out, const Tensor& ids, const Tensor& table) {
+  DLIA_ON_DEVICE_OF(out);
+  check_f32(out, "out"); check_i32(ids, "ids"); check_act(table, "table");
+  DLIA_CHECK(out.dim() == 2 && table.dim() == 2 && table.is_contiguous() && out.size(1) == table.size(1) &&
+             ids.numel() == out.size(0), "embed32: out [T, H], ids [T], table [V, H]");
+  dlia_embed32(out.data_ptr<float>(), ids.data_ptr<int>(), table.data_ptr(), is_f32(table), (int)out.size(0), (int)out.size(1),
+               (int)table.size(0), cur_stream());
+}
+
+void norm32(const std::optional<Tensor>& out, Tensor x, OptTensor y, OptTensor wb, OptTensor wn, OptTensor row_idx, double eps,
+            double off) {
+  DLIA_ON_DEVICE_OF(x);
+  check_f32(x, "x"); check_mat(x, "x");
+  const int64_t H = x.size(1);
+  int64_t rows = x.size(0);
+  const int* ridx = nullptr;
+  if (row_idx.has_value()) {
+    check_i32(*row_idx, "row_idx");
+    DLIA_CHECK(!y.has_value(), "norm32: gathered rows take no addend");
+    rows = row_idx->numel(); ridx = row_idx->data_ptr<int>();
+  }
+  const float* yp = nullptr; long ldy = 0;
+  if (y.has_value()) {
+    check_f32(*y, "y"); check_mat(*y, "y");
+    DLIA_CHECK(y->size(0) >= rows && y->size(1) == H && wb.has_value(), "norm32: y [rows, H] with its weight");
+    yp = y->data_ptr<float>(); ldy = y->stride(0);
+  }
+  void* op = nullptr; long ldo = 0; int of32 = 1;
+  if (out.has_value()) {
+    check_act(*out, "out"); check_mat(*out, "out");
+    DLIA_CHECK(out->size(0) >= rows && out->size(1) == H && wn.has_value(), "norm32: out [rows, H] with its weight");
+    op = out->data_ptr(); ldo = out->stride(0); of32 = is_f32(*out);
+  }
+  DLIA_CHECK(op || yp, "norm32: nothing to do");
+  dlia_norm32(op, of32, x.data_ptr<float>(), yp, opt_f32(wb, H, "wb"), opt_f32(wn, H, "wn"), ridx, (int)rows, (int)H,
+              x.stride(0), ldy, ldo, (float)eps, (float)off, cur_stream());
+}
+
+void gated_headnorm(Tensor out, const Tensor& o, const Tensor& gate, const Tensor& w, int64_t heads, int64_t dv, double eps) {
+  DLIA_ON_DEVICE_OF(out);
+  check_act(out, "out"); check_mat(out, "out"); check_mat(o, "o"); check_mat(gate, "gate"); check_f32(w, "w");
+  DLIA_CHECK(o.scalar_type() == at::kFloat && gate.scalar_type() == at::kFloat && o.is_cuda() && gate.is_cuda(), "o, gate: float32");
+  const int64_t T = out.size(0);
+  DLIA_CHECK(o.size(0) >= T && gate.size(0) >= T && out.size(1) == heads * dv && o.size(1) == heads * dv &&
+             gate.size(1) == heads * dv && w.numel() == dv, "gated_headnorm: shapes");
+  dlia_gated_headnorm(out.data_ptr(), is_f32(out), o.data_ptr<float>(), gate.data_ptr<float>(), w.data_ptr<float>(), (int)T,
+                      (int)heads, (int)dv, o.stride(0), gate.stride(0), out.stride(0), (float)eps, cur_stream());
+}
+
+void gemm_any(Tensor out, const Tensor& x, const Tensor& w, OptTensor bias, int64_t epi) {
+  DLIA_ON_DEVICE_OF(out);
+  check_act(out, "out"); check_act(x, "x"); check_act(w, "w");
+  check_mat(out, "out"); check_mat(x, "x"); check_mat(w, "w");
+  DLIA_CHECK(x.scalar_type() == w.scalar_type(), "gemm_any: x and w must have one type");
+  DLIA_CHECK(is_f32(out) || !is_f32(x), "gemm_any: fp32 operands give fp32 output");
+  const int64_t M = x.size(0), K = x.size(1), N = w.size(0);
+  DLIA_CHECK(w.size(1) == K && out.size(0) >= M, "gemm_any: x [M, K], w [N, K], out [M, .]");
+  DLIA_CHECK(epi == 0 || epi == 1, "gemm_any: epi 0 or 1");
+  if (epi == 0) {
+    DLIA_CHECK(out.size(1) == N, "gemm_any: out [M, N]");
+  } else {
+    DLIA_CHECK(N % 32 == 0 && out.size(1) == N / 2, "gemm_any: gated output is [M, N / 2], N a multiple of 32");
+  }
+  dlia_gemm_any(out.data_ptr(), is_f32(out), x.data_ptr(), w.data_ptr(), is_f32(x), opt_f32(bias, N, "bias"), (int)M, (int)N,
+                (int)K, x.stride(0), w.stride(0), out.stride(0), (int)epi, cur_stream());
+}
+
+void gated_gelu(Tensor act, const Tensor& gu) {
+  DLIA_ON_DEVICE_OF(act);
+  check_bf16(act, "act"); check_bf16(gu, "gu"); check_rows(act, "act"); check_rows(gu, "gu");
+  const int64_t M = act.size(0), F = act.size(1);
+  DLIA_CHECK(gu.size(0) >= M && gu.size(1) == 2 * F && F % 8 == 0, "gated_gelu: gu [M, 2F], act [M, F], F a multiple of 8");
+  dlia_gated_gelu(act.data_ptr(), gu.data_ptr(), (int)M, (int)F, gu.stride(0), act.stride(0), cur_stream());
+}
+
+static void check_paged(const Tensor& kc, const Tensor& vc, const Tensor& tok_pos, const Tensor& tok_seq, const Tensor& table,
+                        int64_t T, int64_t G, int64_t d, int64_t dv) {
+  check_act(kc, "kcache"); check_act(vc, "vcache");
+  DLIA_CHECK(kc.scalar_type() == vc.scalar_type() && kc.is_contiguous() && vc.is_contiguous(), "caches: one type, contiguous");
+  DLIA_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.size(0) == vc.size(0) && kc.size(1) == G && vc.size(1) == G &&
+             kc.size(2) == 32 && vc.size(2) == 32 && kc.size(3) == d && vc.size(3) == dv, "caches: [blocks, G, 32, d | dv]");
+  check_i32(tok_pos, "tok_pos"); check_i32(tok_seq, "tok_seq"); check_i32(table, "block_table");
+  DLIA_CHECK(tok_pos.numel() >= T && tok_seq.numel() >= T && table.dim() == 2, "per-token metadata / block table shape");
+  DLIA_CHECK(d >= 1 && d <= 512 && dv >= 1 && dv <= 512 && G >= 1, "head sizes 1..512");
+}
+
+void kv_store(const Tensor& qkv, const std::optional<Tensor>& vfirst, OptTensor lam, int64_t mix, Tensor kcache, Tensor vcache,
+              const Tensor& tok_pos, const Tensor& tok_seq, const Tensor& block_table, int64_t G, int64_t d, int64_t dv,
+              int64_t q_cols) {
+  DLIA_ON_DEVICE_OF(kcache);
+  check_mat(qkv, "qkv");
+  DLIA_CHECK(qkv.is_cuda() && qkv.scalar_type() == at::kFloat, "qkv: float32");
+  const int64_t T = qkv.size(0);
+  DLIA_CHECK(qkv.size(1) == q_cols + G * (d + dv), "kv_store: qkv [T, q + k + v]");
+  check_paged(kcache, vcache, tok_pos, tok_seq, block_table, T, G, d, dv);
+  DLIA_CHECK(mix >= 0 && mix <= 2, "mix 0..2");
+  float* vf = nullptr;
+  if (mix) {
+    DLIA_CHECK(vfirst.has_value(), "value mixing needs the buffer of first values");
+    check_f32(*vfirst, "vfirst");
+    DLIA_CHECK(vfirst->numel() >= T * G * dv, "vfirst too small");
+    vf = vfirst->data_ptr<float>();
+  }
+  const float* lp = opt_f32(lam, 1, "lam");
+  DLIA_CHECK(mix != 2 || lp, "mix 2 needs lam");
+  dlia_kv_store(qkv.data_ptr<float>(), vf, lp, (int)mix, kcache.data_ptr(), vcache.data_ptr(), is_f32(kcache),
+                tok_pos.data_ptr<int>(), tok_seq.data_ptr<int>(), block_table.data_ptr<int>(), (int)T, (int)block_table.size(1),
+                (int)kcache.size(0), (int)block_table.size(0), (int)G, (int)d, (int)dv, (int)q_cols, qkv.stride(0), cur_stream());
+}
+
+void window_attention(Tensor out, const Tensor& qkv, const Tensor& kcache, const Tensor& vcache, const Tensor& tok_pos,
+                      const Tensor& tok_seq, const Tensor& block_table, int64_t H, int64_t G, int64_t d, int64_t dv, double scale,
+                      int64_t window, bool sink) {
+  DLIA_ON_DEVICE_OF(out);
+  check_act(out, "out"); check_mat(out, "out"); check_mat(qkv, "qkv");
+  DLIA_CHECK(qkv.is_cuda() && qkv.scalar_type() == at::kFloat, "qkv: float32");
+  const int64_t T = out.size(0);
+  DLIA_CHECK(qkv.size(0) >= T && qkv.size(1) >= H * d && out.size(1) == H * dv && H % G == 0, "window_attention: shapes");
+  check_paged(kcache, vcache, tok_pos, tok_seq, block_table, T, G, d, dv);
+  DLIA_CHECK(out.scalar_type() == kcache.scalar_type(), "window_attention: output in the cache's type");
+  dlia_window_attention(out.data_ptr(), qkv.data_ptr<float>(), kcache.data_ptr(), vcache.data_ptr(), is_f32(kcache),
+                        tok_pos.data_ptr<int>(), tok_seq.data_ptr<int>(), block_table.data_ptr<int>(), (int)T,
+                        (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0), (int)H, (int)G, (int)d, (int)dv,
+                        qkv.stride(0), out.stride(0), (float)scale, (int)window, sink ? 1 : 0, cur_stream());
+}
+
+void short_conv(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, const Tensor& q_start, const Tensor& ctx,
+                const Tensor& slots, int64_t max_q) {
+  DLIA_ON_DEVICE_OF(y);
+  check_f32(y, "y"); check_f32(carry, "carry"); check_f32(taps, "taps"); check_mat(z, "z");
+  DLIA_CHECK(z.is_cuda() && z.scalar_type() == at::kFloat, "z: float32");
+  check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots");
+  const int64_t B = ctx.numel(), C = taps.size(0), K = taps.size(1);
+  DLIA_CHECK(taps.dim() == 2 && K >= 1 && K <= 16, "short_conv: 1..16 taps");
+  DLIA_CHECK(y.dim() == 2 && y.size(1) == C && z.size(1) >= C && z.size(0) >= y.size(0), "short_conv: y [T, C], z [T, >= C]");
+  DLIA_CHECK(q_start.numel() >= B + 1 && slots.numel() >= B, "short_conv: q_start [B + 1], ctx [B], slots [B]");
+  DLIA_CHECK(carry.dim() == 3 && carry.size(1) == std::max<int64_t>(K - 1, 1) && carry.size(2) == C, "short_conv: carry [slots, K - 1, C]");
+  DLIA_CHECK(max_q <= y.size(0), "short_conv: max_q beyond the step's tokens");
+  dlia_short_conv(y.data_ptr<float>(), z.data_ptr<float>(), carry.data_ptr<float>(), taps.data_ptr<float>(), q_start.data_ptr<int>(),
+                  ctx.data_ptr<int>(), slots.data_ptr<int>(), (int)B, (int)max_q, (int)C, (int)K, z.stride(0), (int)carry.size(0),
+                  cur_stream());
+}
+
+void unit_heads(Tensor x, int64_t heads, int64_t d, int64_t scaled_heads, double mult, double eps) {
+  DLIA_ON_DEVICE_OF(x);
+  check_mat(x, "x");
+  DLIA_CHECK(x.scalar_type() == at::kFloat && x.size(1) == heads * d, "unit_heads: x [T, heads * d] float32");
+  dlia_unit_heads(x.data_ptr<float>(), (int)x.size(0), (int)heads, (int)d, x.stride(0), (int)scaled_heads, (float)mult, (float)eps,
+                  cur_stream());
+}
+
+void delta_rule(Tensor o, const Tensor& y, const Tensor& z, Tensor state, const Tensor& A_log, const Tensor& dt_bias,
+                const Tensor& q_start, const Tensor& ctx, const Tensor& slots, int64_t G, int64_t Hv, int64_t d, int64_t dv,
+                int64_t col_beta, int64_t col_a, int64_t max_q) {
+  DLIA_ON_DEVICE_OF(o);
+  check_f32(o, "o"); check_f32(y, "y"); check_f32(state, "state"); check_f32(A_log, "A_log"); check_f32(dt_bias, "dt_bias");
+  check_mat(z, "z");
+  DLIA_CHECK(z.is_cuda() && z.scalar_type() == at::kFloat, "z: float32");
+  check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots");
+  const int64_t B = ctx.numel(), C = 2 * G * d + Hv * dv, T = y.size(0);
+  DLIA_CHECK(Hv % G == 0 && y.dim() == 2 && y.size(1) == C && o.dim() == 2 && o.size(0) >= T && o.size(1) == Hv * dv, "delta_rule: y [T, C], o [T, Hv dv]");
+  DLIA_CHECK(z.size(0) >= T && col_beta + Hv <= z.size(1) && col_a + Hv <= z.size(1) && col_beta >= 0 && col_a >= 0, "delta_rule: gate columns");
+  DLIA_CHECK(state.dim() == 4 && state.size(1) == Hv && state.size(2) == d && state.size(3) == dv, "delta_rule: state [slots, Hv, d, dv]");
+  DLIA_CHECK(A_log.numel() == Hv && dt_bias.numel() == Hv && q_start.numel() >= B + 1 && slots.numel() >= B, "delta_rule: per-head / per-sequence vectors");
+  const int rc = dlia_delta_rule(o.data_ptr<float>(), y.data_ptr<float>(), z.data_ptr<float>(), state.data_ptr<float>(),
+                                 A_log.data_ptr<float>(), dt_bias.data_ptr<float>(), q_start.data_ptr<int>(), ctx.data_ptr<int>(),
+                                 slots.data_ptr<int>(), (int)B, (int)G, (int)Hv, (int)d, (int)dv, (int)C, z.stride(0), (int)col_beta,
+                                 (int)col_a, (int)state.size(0), (int)max_q, cur_stream());
+  DLIA_CHECK(rc == 0, "delta_rule: key size ", d, " is beyond what the kernel holds in registers (512)");
+}
+
 }  // namespace
 
 TORCH_LIBRARY(dlia, m) {
+  m.def("embed32(Tensor(a!) out, Tensor ids, Tensor table) -> ()");
+  m.def("norm32(Tensor(a!)? out, Tensor(b!) x, Tensor? y, Tensor? wb, Tensor? wn, Tensor? row_idx, float eps, float off) -> ()");
+  m.def("gated_headnorm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, int heads, int dv, float eps) -> ()");
+  m.def("gated_gelu(Tensor(a!) act, Tensor gu) -> ()");
+  m.def("paged_attention_window(Tensor(a!) out, Tensor qkv, Tensor kv_cache, Tensor q_start, Tensor ctx_lens, Tensor block_table, Tensor? slots, Tensor? partial, int max_q_len, int Hq, int Hkv, int D, float scale, int splits, int window, bool sink) -> ()");
+  m.def("value_mix(Tensor(a!) qkv, Tensor(b!) vfirst, Tensor? lam, int mix, int v_off, int v_cols) -> ()");
+  m.def("gemm_any(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, int epi) -> ()");
+  m.def("kv_store(Tensor qkv, Tensor(a!)? vfirst, Tensor? lam, int mix, Tensor(b!) kcache, Tensor(c!) vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int G, int d, int dv, int q_cols) -> ()");
+  m.def("window_attention(Tensor(a!) out, Tensor qkv, Tensor kcache, Tensor vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int G, int d, int dv, float scale, int window, bool sink) -> ()");
+  m.def("short_conv(Tensor(a!) y, Tensor z, Tensor(b!) carry, Tensor taps, Tensor q_start, Tensor ctx, Tensor slots, int max_q) -> ()");
+  m.def("unit_heads(Tensor(a!) x, int heads, int d, int scaled_heads, float mult, float eps) -> ()");
+  m.def("delta_rule(Tensor(a!) o, Tensor y, Tensor z, Tensor(b!) state, Tensor A_log, Tensor dt_bias, Tensor q_start, Tensor ctx, Tensor slots, int G, int Hv, int d, int dv, int col_beta, int col_a, int max_q) -> ()");
   m.def("norm(Tensor(a!) out, Tensor(b!) x, Tensor? delta, Tensor? partial, int splits, Tensor? pbias, Tensor w, Tensor? b, Tensor? row_idx, float eps, int mode) -> ()");
   m.def("embed(Tensor(a!) out, Tensor ids, Tensor? pos, Tensor wte, Tensor? wpe) -> ()");
   m.def("rope_kvwrite(Tensor(a!) qkv, Tensor? partial, int splits, Tensor? pbias, Tensor(b!) kv_cache, Tensor cos, Tensor sin, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int Hq, int Hkv, int D, bool use_rope) -> ()");
@@ -657,6 +879,18 @@ TORCH_LIBRARY(dlia, m) {
 }
 
 TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
+  m.impl("embed32", &embed32);
+  m.impl("norm32", &norm32);
+  m.impl("gated_headnorm", &gated_headnorm);
+  m.impl("gemm_any", &gemm_any);
+  m.impl("gated_gelu", &gated_gelu);
+  m.impl("paged_attention_window", &paged_attention_window);
+  m.impl("value_mix", &value_mix);
+  m.impl("kv_store", &kv_store);
+  m.impl("window_attention", &window_attention);
+  m.impl("short_conv", &short_conv);
+  m.impl("unit_heads", &unit_heads);
+  m.impl("delta_rule", &delta_rule);
   m.impl("norm", &norm);
   m.impl("embed", &embed);
   m.impl("rope_kvwrite", &rope_kvwrite);

@@ -85,7 +85,9 @@ void dlia_paged_attention(void* out, const void* qkv, const void* kv_cache, cons
                           const int* q_start, const int* ctx_lens, const int* block_table,
                           const int* slots, float* partial, int B, int max_q_len, int Hq,
                           int Hkv, int D, int table_rows, int max_blocks, int num_blocks,
-                          long ldq, long ldo, float scale, int splits, hipStream_t stream);
+                          long ldq, long ldo, float scale, int splits, hipStream_t stream, int window = 0, int sink = 0);
+// (window > 0: a query at i sees the keys j with 0 <= i - j < window; sink: one more softmax term exp(0) without a value;
+// both for the bf16 cache only)
 long dlia_paged_attention_ws_floats(int B, int max_q_len, int Hq, int Hkv, int D, int splits);
 
 // ---- sampler.hip ----------------------------------------------------------------------
@@ -98,6 +100,43 @@ void dlia_sample(int* out_tokens, const float* logits, const float* temperature,
                  const int* steps, int R, int vocab, long ldl, float* dbg_probs,
                  int* dbg_ids, int dbg_cap, hipStream_t stream, const float* chunk_max = nullptr, long ldc = 0,
                  int* ids_out = nullptr, int* steps_adv = nullptr, int* ctx_adv = nullptr);
+
+// ---- norm32.hip (fp32 residual stream) ------------------------------------------------------
+void dlia_embed32(float* out, const int* ids, const void* table, int table_f32, int T, int H, int vocab, hipStream_t stream);
+// y != null: x += rms(y) * (off + wb); out != null: out = rms(x[row_idx ? row_idx[r] : r]) * (off + wn)
+void dlia_norm32(void* out, int out_f32, float* x, const float* y, const float* wb, const float* wn, const int* row_idx,
+                 int rows, int H, long ldx, long ldy, long ldo, float eps, float off, hipStream_t stream);
+void dlia_gated_headnorm(void* out, int out_f32, const float* o, const float* gate, const float* w, int T, int heads, int dv,
+                         long ldo_in, long ldg, long ld_out, float eps, hipStream_t stream);
+
+// ---- gemm_any.hip ---------------------------------------------------------------------------
+// C[M,N] = A[M,K] . W[N,K]^T (+ bias), any shape, row-major W; epi 1: gated pair (interleaved gate / up tiles) ->
+// gelu_tanh(gate) * up, N / 2 columns
+void dlia_gemm_any(void* C, int out_f32, const void* A, const void* W, int in_f32, const float* bias, int M, int N, int K,
+                   long lda, long ldw, long ldc, int epi, hipStream_t stream);
+
+// act[m, j] = gelu_tanh(gu[m, j]) * gu[m, F + j] (bf16, F a multiple of 8, 16-byte aligned rows)
+void dlia_gated_gelu(void* act, const void* gu, int M, int F, long ldg, long lda, hipStream_t stream);
+
+// ---- window_attention.hip -------------------------------------------------------------------
+void dlia_kv_store(const float* qkv, float* vfirst, const float* lam, int mix, void* kcache, void* vcache, int cache_f32,
+                   const int* tok_pos, const int* tok_seq, const int* block_table, int T, int max_blocks, int num_blocks,
+                   int table_rows, int G, int d, int dv, int q_cols, long ld, hipStream_t stream);
+void dlia_window_attention(void* out, const float* qkv, const void* kcache, const void* vcache, int f32, const int* tok_pos,
+                           const int* tok_seq, const int* block_table, int T, int max_blocks, int num_blocks, int table_rows,
+                           int H, int G, int d, int dv, long ldq, long ldo, float scale, int window, int sink,
+                           hipStream_t stream);
+
+// v <- (1 - lam) v + lam v_first on the v columns of a bf16 fused qkv activation (mix 2), or v_first <- v (mix 1)
+void dlia_value_mix(void* qkv, float* vfirst, const float* lam, int mix, int T, int v_off, int v_cols, long ld, hipStream_t stream);
+
+// ---- delta_rule.hip -------------------------------------------------------------------------
+void dlia_short_conv(float* y, const float* z, float* carry, const float* taps, const int* q_start, const int* ctx,
+                     const int* slots, int B, int max_q, int C, int K, long ldz, int state_rows, hipStream_t stream);
+void dlia_unit_heads(float* x, int T, int heads, int d, long ld, int scaled_heads, float mult, float eps, hipStream_t stream);
+int dlia_delta_rule(float* o, const float* y, const float* z, float* state, const float* A_log, const float* dt_bias,
+                    const int* q_start, const int* ctx, const int* slots, int B, int G, int Hv, int d, int dv, int C, long ldz,
+                    int col_beta, int col_a, int state_rows, int max_q, hipStream_t stream);
 
 // ---- misc.hip -------------------------------------------------------------------------
 void dlia_advance_i32(int* x, int n, int delta, hipStream_t stream);
