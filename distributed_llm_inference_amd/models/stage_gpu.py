@@ -146,22 +146,12 @@ class GpuStage:
         self.kv8 = kv_dtype == "fp8"
         self.decode_rows = int(decode_rows if decode_rows is not None else os.environ.get("DLIA_DECODE_ROWS", DEFAULT_DECODE_ROWS))
         self._guided_ok = os.environ.get("DLIA_GUIDED_SAMPLER", "1") != "0"      # A/B switch: 0 = the sampler reads whole rows
-        self.K = ops.load()
         # decoder-layer GEMMs: "fp8" = e4m3 weights (per-channel scale) x e4m3 activations (per-row
         # dynamic scale) on the block-scaled fp8 MFMA; "fp8w" = e4m3 weights widened to bf16 in
         # registers, bf16 activations
         self.wmode = weight_dtype
         self.w8 = weight_dtype != "bf16"
-        self.spec, self.plan = spec, plan
-        self.device = torch.device(device)
-        self.max_slots, self.max_seq_len = max_slots, max_seq_len
-        self.max_blocks = (max_seq_len + BLOCK - 1) // BLOCK
-        self.max_tokens = max(max_tokens, max_batch)
-        self.max_batch = max_batch
-        # row counts a micro-batch may run its fixed-shape decode step at (ascending, max_batch last)
-        self.graph_sizes = sorted({int(b) for b in (graph_sizes or []) if 0 < int(b) < max_batch}) + [max_batch]
-        self.use_graphs = use_graphs
-        self.null_slot = max_slots            # extra block-table row that never owns blocks
+        self._init_limits(spec, plan, device, max_slots, max_seq_len, max_tokens, max_batch, use_graphs, graph_sizes)
         dev, bf = self.device, torch.bfloat16
         H, I, V = spec.hidden_size, spec.intermediate_size, spec.vocab_size
 
@@ -216,25 +206,45 @@ class GpuStage:
         self._ws_floats = need
         self._gemm_shapes = [(spec.qkv_size, H), (H, spec.q_size), (H, I), (2 * I if spec.is_llama else I, H)]
         self.wk0 = self._new_work(self.max_tokens)
-        # step metadata: pinned staging ring (host) and one landing buffer per stream (device)
+        # ---- paged KV cache for this stage's layers ---------------------------------------
+        # (after the workspaces: the cache takes what is left of the device)
+        self._init_step_state(kv_mem_fraction, decode_states)
+        if not defer_kv:
+            self.allocate_kv(num_blocks if num_blocks is not None else self.kv_budget_blocks())
+        self._gemm_cfg: Dict[tuple, tuple] = {}
+        self._ones = torch.ones(H, device=dev, dtype=bf)
+        self.scale = 1.0 / math.sqrt(spec.head_dim)
+
+    def _init_limits(self, spec, plan, device, max_slots, max_seq_len, max_tokens, max_batch, use_graphs, graph_sizes):
+        """What every executor on this library shares, whatever its layers are: the kernel library, the
+        step limits, the block-table geometry, the fixed-shape decode sizes."""
+        self.K = ops.load()
+        self.spec, self.plan = spec, plan
+        self.device = torch.device(device)
+        self.max_slots, self.max_seq_len = max_slots, max_seq_len
+        self.max_blocks = (max_seq_len + BLOCK - 1) // BLOCK
+        self.max_tokens = max(max_tokens, max_batch)
+        self.max_batch = max_batch
+        # row counts a micro-batch may run its fixed-shape decode step at (ascending, max_batch last)
+        self.graph_sizes = sorted({int(b) for b in (graph_sizes or []) if 0 < int(b) < max_batch}) + [max_batch]
+        self.use_graphs = use_graphs
+        self.null_slot = max_slots            # extra block-table row that never owns blocks
+
+    def _init_step_state(self, kv_mem_fraction: float, decode_states: int):
+        """Step metadata staging (pinned ring on the host, one landing buffer per stream on the device),
+        the block table, and the books of the fixed-shape decode states."""
+        dev = self.device
         self._table_cap = 1 << 16                   # words of one block-table upload; larger updates go in pieces
-        self._md_words = 3 * self.max_tokens + 16 * max_batch + 64
+        self._md_words = 4 * self.max_tokens + 16 * self.max_batch + 64
         self._ring = _PinnedRing(max(self._md_words, self._table_cap))
         self._landing: Dict[int, torch.Tensor] = {}
         self._eager_sampling = None                 # (step id, device views) staged by `forward` for `sample`
-        # ---- paged KV cache for this stage's layers ---------------------------------------
-        # (after the workspaces: the cache takes what is left of the device)
         self.kv_mem_fraction, self.decode_states = kv_mem_fraction, max(1, decode_states)
         self.kv = self.kv_scale = None
         self.num_blocks = 0
-        self.block_table = torch.full((max_slots + 1, self.max_blocks), -1, device=dev, dtype=torch.int32)
-        if not defer_kv:
-            self.allocate_kv(num_blocks if num_blocks is not None else self.kv_budget_blocks())
+        self.block_table = torch.full((self.max_slots + 1, self.max_blocks), -1, device=dev, dtype=torch.int32)
         self._mbs: Dict[tuple, _MicroBatchState] = {}      # (micro-batch, rows) -> static decode state
-        self._gemm_cfg: Dict[tuple, tuple] = {}
-        self._ones = torch.ones(H, device=dev, dtype=bf)
-        self._arange = torch.arange(max_batch + 1, device=dev, dtype=torch.int32)      # q_start of a decode step: one token per row
-        self.scale = 1.0 / math.sqrt(spec.head_dim)
+        self._arange = torch.arange(self.max_batch + 1, device=dev, dtype=torch.int32)      # q_start of a decode step: one token per row
         self.graph_replays = 0
         self.graph_captures = 0
 
@@ -424,6 +434,10 @@ class GpuStage:
         ok = [s for s in slots if 0 <= s < self.max_slots]
         self._write_table_rows(ok, [[]] * len(ok))
 
+    def _embed_rows(self, wk, T: int, ids, pos):
+        """wk.h[:T] <- embedding rows of `ids` (plus the learned position rows where the family has them)."""
+        self.K.embed(wk.h[:T], ids, pos, self.embed, self.pos_embed)
+
     # ---- the layer stack on T tokens ------------------------------------------------------
     def _cfg(self, M: int, N: int, K: int, epi: int):
         key = (M, N, K, epi)
@@ -569,9 +583,15 @@ class GpuStage:
         tok_seq = np.repeat(slots, q)
         tok_pos = (np.arange(T, dtype=np.int64) - np.repeat(q_start[:-1] - c, q)).astype(np.int32)
         sampled = (np.asarray(batch.sample, dtype=np.int64) != 0) & (q > 0)
-        rows = (q_start[1:][sampled] - 1).astype(np.int32)
+        scoring = batch.score_rows is not None      # logits of the named token rows instead of a token per sequence
+        if scoring:
+            rows = np.asarray(batch.score_rows, dtype=np.int32)
+            if rows.size and (int(rows.min()) < 0 or int(rows.max()) >= T):
+                raise ValueError("score_rows must index the step's tokens")
+        else:
+            rows = (q_start[1:][sampled] - 1).astype(np.int32)
         R = int(rows.size)
-        if R > self.max_batch:
+        if R > self.max_batch and not scoring:
             raise ValueError(f"{R} sampled rows exceed max_batch {self.max_batch}")
         dev = self.device
         parts = [tok_pos, tok_seq, q_start.astype(np.int32), c.astype(np.int32), slots, rows]
@@ -582,7 +602,7 @@ class GpuStage:
             if ids_h.size != T:
                 raise ValueError(f"expected {T} token ids, got {ids_h.size}")
             parts.append(ids_h)
-        if self.plan.has_head and R:
+        if self.plan.has_head and R and not scoring:
             pick = lambda vals, dt: np.asarray(vals, dtype=dt)[sampled]
             parts += [pick(batch.temperature, np.float32), pick(batch.top_k, np.int32), pick(batch.top_p, np.float32),
                       pick(batch.sample_steps, np.int32), pick(batch.seeds, np.int64)]
@@ -597,12 +617,12 @@ class GpuStage:
                 ids = x.to(dtype=torch.int32).reshape(-1)
                 if ids.numel() != T:
                     raise ValueError(f"expected {T} token ids, got {ids.numel()}")
-            self.K.embed(wk.h[:T], ids, md_tok_pos, self.embed, self.pos_embed)
+            self._embed_rows(wk, T, ids, md_tok_pos)
         else:
             if tuple(x.shape) != (T, s.hidden_size):
                 raise ValueError(f"expected hidden [{T},{s.hidden_size}], got {tuple(x.shape)}")
             wk.h[:T].copy_(x.to(device=dev, dtype=torch.bfloat16), non_blocking=True)
-        self._eager_sampling = (batch.step_id, R, up[nxt:nxt + 5]) if (self.plan.has_head and R) else None
+        self._eager_sampling = (batch.step_id, R, up[nxt:nxt + 5]) if (self.plan.has_head and R and not scoring) else None
         max_q = int(q.max()) if B else 1
         lead = 0                                   # decode tokens riding in front of prompt chunks (Engine._submit_prefill)
         if max_q > 1:
@@ -615,6 +635,13 @@ class GpuStage:
             return wk.h[:T]
         if R == 0:
             return wk.logits[:0, :s.vocab_size]
+        if scoring:
+            # any number of rows: the head runs over as many as its workspace holds at a time, the logits are copied out
+            out = torch.empty(R, s.vocab_size, device=dev, dtype=torch.float32)
+            for i in range(0, R, self.max_batch):
+                n = min(self.max_batch, R - i)
+                out[i:i + n] = self._head(wk, md_rows[i:i + n], n, T, pend)[:, :s.vocab_size]
+            return out
         return self._head(wk, md_rows, R, T, pend)[:, :s.vocab_size]
 
     @torch.no_grad()
@@ -674,7 +701,7 @@ class GpuStage:
         """One decode step over the micro-batch's static buffers (captured into the graph)."""
         K, B, wk = self.K, st.B, st.wk
         if self.plan.has_embed:
-            K.embed(wk.h[:B], st.ids, st.ctx, self.embed, self.pos_embed)
+            self._embed_rows(wk, B, st.ids, st.ctx)
         else:
             wk.h[:B].copy_(st.hidden_in)
         pend = self._layers(wk, B, B, st.ctx, st.slots, self._arange[:B + 1], st.ctx, st.slots, 1, st.splits)

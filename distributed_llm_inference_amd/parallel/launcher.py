@@ -71,7 +71,7 @@ def ctrl_slot_bytes(cfg: EngineConfig) -> int:
     per_seq_blocks = (cfg.max_seq_len + 31) // 32
     chunk = max(cfg.prefill_chunk, cfg.max_batch)
     n = 64 + 40 * cfg.max_batch + 4 * chunk + 4 * (2 * cfg.max_batch + chunk // 32 + per_seq_blocks + cfg.max_batch) \
-        + 12 * cfg.max_batch + 4096 \
+        + 12 * cfg.max_batch + 4096 + 4 * chunk + 8 \
         + 4 * Engine.MOVE_BUDGET + 8 * min(cfg.max_batch, Engine.MOVE_BUDGET)      # tables of rows moved at a recomposition
     size = 1 << 16
     while size < n:
@@ -93,7 +93,20 @@ def build_executor(cfg: EngineConfig, spec: ModelSpec, plan: StagePlan, device: 
     `defer_kv` the cache is allocated later by `settle_kv` (the stages first agree on one count)."""
     backend = cfg.resolved_backend()
     dev = device or cfg.resolved_device()
+    if backend == "hip" and spec.is_hybrid:
+        # models described layer by layer (windowed attention, recurrent mixers, fp32 residual stream)
+        from ..models.stage_hybrid import HybridGpuStage
+        if cfg.dtype not in ("bf16", "fp32") or cfg.kv_dtype != "bf16":
+            raise ValueError(f"{spec.name}: hybrid stacks run in bf16 or fp32 with a cache of the same type")
+        w = load_weights(cfg, spec, plan, dev, torch.float32 if cfg.dtype == "fp32" else torch.bfloat16)
+        return HybridGpuStage(spec, plan, w, device=dev, max_slots=cfg.num_micro_batches * cfg.max_batch,
+                              max_seq_len=cfg.max_seq_len, num_blocks=cfg.kv_blocks if cfg.kv_blocks > 0 else None,
+                              max_tokens=cfg.prefill_chunk, max_batch=cfg.max_batch, use_graphs=cfg.use_graphs,
+                              kv_mem_fraction=cfg.kv_mem_fraction, dtype=cfg.dtype, decode_states=cfg.num_micro_batches,
+                              defer_kv=defer_kv, graph_sizes=cfg.graph_sizes())
     if backend == "hip":
+        if cfg.dtype == "fp32":
+            raise ValueError(f"{spec.name}: the HIP executor of this family has no fp32 mode (bf16, fp8, fp8w)")
         from ..models.stage_gpu import GpuStage
         w = load_weights(cfg, spec, plan, dev, torch.bfloat16)
         return GpuStage(spec, plan, w, device=dev, max_slots=cfg.num_micro_batches * cfg.max_batch,
