@@ -6,6 +6,7 @@
     generate  one prompt through a local in-process engine
     bench     the headline decode benchmark (same as bench.py)
     plan      print the layer partition for a model / stage count
+    trace     replay a trace of token ids (JSON lines on stdin) step by step and write the logits asked for
 """
 from __future__ import annotations
 
@@ -103,6 +104,14 @@ def main(argv=None) -> int:
     p.add_argument("--temperature", type=float, default=None)
     p = sub.add_parser("plan"); _add_engine_args(p)
     p = sub.add_parser("bench"); p.add_argument("rest", nargs=argparse.REMAINDER)
+    p = sub.add_parser("trace", help="replay a trace from stdin: one JSON step per line, logits to --out/<step>.f32")
+    p.add_argument("--model", required=True, help="built-in name or checkpoint directory")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32", "bf16", "fp32"])
+    p.add_argument("--out", required=True, help="directory for the logits files")
+    p.add_argument("--max-tokens", type=int, default=4096, help="tokens the cache pool holds (live requests, each rounded up to whole blocks)")
+    p.add_argument("--slots", type=int, default=4, help="requests that can be live at once")
+    p.add_argument("--backend", default="auto", choices=["auto", "hip", "torch"])
+    p.add_argument("--device", default="auto", choices=["auto", "cuda", "cpu"])
     a = ap.parse_args(argv)
 
     if a.cmd == "serve":
@@ -131,6 +140,9 @@ def main(argv=None) -> int:
             extra = [x for x, on in (("embedding", pl.has_embed), ("final norm + lm_head + sampler", pl.has_head)) if on]
             # x.5 = a boundary between a layer's attention and MLP blocks (`StagePlan.describe`)
             print(f"stage {pl.stage}: layers {pl.describe()}" + (f" + {', '.join(extra)}" if extra else ""))
+    elif a.cmd == "trace":
+        from ..runtime.trace_runner import run
+        return run(a.model, a.dtype, a.out, a.max_tokens, a.slots, device=a.device, backend=a.backend)
     elif a.cmd == "bench":
         import os
         import runpy
