@@ -79,6 +79,10 @@ def parse():
                     help="sequences of the single micro-batch of the low-latency region (0: skip both low-latency regions)")
     ap.add_argument("--latency-steps", type=int, default=24, help="timed steps of each low-latency region")
     ap.add_argument("--no-hop-probe", action="store_true", help="do not time the hops before the run")
+    ap.add_argument("--hybrid-compare", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of Letarax stacks beside Llama stacks "
+                         "of equal size on one GPU (bench/hybrid_compare.py), one JSON line per size")
+    ap.add_argument("--hybrid-sizes", default="", help="with --hybrid-compare: comma-separated size names (default: all)")
     ap.add_argument("--preflight", action="store_true",
                     help="no model: report devices, peer access and RCCL, open + warm + time + close every hop, exit")
     return ap.parse_args()
@@ -386,6 +390,10 @@ def preflight(a, world: int, emit=print) -> int:
 
 def main():
     a = parse()
+    if a.hybrid_compare:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import hybrid_compare
+        raise SystemExit(hybrid_compare.main([x for x in a.hybrid_sizes.split(",") if x] or None))
     env_world = os.environ.get("WORLD_SIZE")
     if env_world is None and a.gpus > 1:
         # no launcher: this process becomes one (it never touches a GPU; nothing below runs in it)
