@@ -21,14 +21,10 @@ VOCAB = 32000
 
 
 def specs(name: str):
-    from distributed_llm_inference_amd.models.spec import LayerSpec, ModelSpec
+    from distributed_llm_inference_amd.models.spec import BUILTIN_SPECS, ModelSpec
     W, H, G, D, F, L, win = SIZES[name]
-    att = LayerSpec("attention", heads=H, kv_heads=G, dim=D, vdim=D, ff=F, window=win, scale=D ** -0.5, sink=True, v_mix=True)
-    dlt = LayerSpec("delta", heads=H, kv_heads=G, dim=D, vdim=D, ff=F, conv=4, scale=D ** -0.5)
-    layers = tuple((att, dlt, att, att)[i % 4] for i in range(L))
-    hyb = ModelSpec(name=f"letarax-{name}", family="letarax", num_layers=L, hidden_size=W, num_heads=H, num_kv_heads=G,
-                    head_dim=D, intermediate_size=F, vocab_size=VOCAB, max_position=1 << 30, norm_eps=1e-5,
-                    tie_embeddings=True, hf_type="letarax", layer_specs=layers)
+    hyb = BUILTIN_SPECS[f"letarax-{name}"]
+    assert (hyb.hidden_size, hyb.num_heads, hyb.num_kv_heads, hyb.head_dim, hyb.intermediate_size, hyb.num_layers) == (W, H, G, D, F, L)
     llama = ModelSpec(name=f"llama-{name}", family="llama", num_layers=L, hidden_size=W, num_heads=H, num_kv_heads=G,
                       head_dim=D, intermediate_size=F, vocab_size=VOCAB, max_position=8192, norm_eps=1e-5, tie_embeddings=True)
     return hyb, llama

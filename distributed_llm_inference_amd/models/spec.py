@@ -504,6 +504,24 @@ BUILTIN_SPECS["llama3-70b"] = BUILTIN_SPECS["llama-3-70b"]
 BUILTIN_SPECS["meta-llama-3-70b"] = BUILTIN_SPECS["llama-3-70b"]
 
 
+def letarax_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int, ff: int, num_layers: int, window: int,
+                 vocab_size: int = 32000, conv: int = 4, pattern: str = "adaa") -> ModelSpec:
+    """A Letarax stack from a few numbers: `pattern` repeats over the layers ('a' windowed attention with the sink and
+    value mixing, 'd' gated delta rule), every layer with a feed-forward of `ff`, keys and values of `head_dim`."""
+    att = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, ff=ff, window=window,
+                    scale=head_dim ** -0.5, sink=True, v_mix=True)
+    dlt = LayerSpec("delta", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, ff=ff, conv=conv, scale=head_dim ** -0.5)
+    layers = tuple(att if pattern[i % len(pattern)] == "a" else dlt for i in range(num_layers))
+    return ModelSpec(name=name, family="letarax", num_layers=num_layers, hidden_size=width, num_heads=heads, num_kv_heads=kv_heads,
+                     head_dim=head_dim, intermediate_size=ff, vocab_size=vocab_size, max_position=1 << 30, norm_eps=1e-5,
+                     tie_embeddings=True, bos_token_id=1, eos_token_id=2, hf_type="letarax", layer_specs=layers)
+
+
+# Letarax stacks of the sizes of the Llama benchmark shapes (random weights; `bench.py --hybrid-compare` runs them)
+BUILTIN_SPECS["letarax-1b-like"] = letarax_spec("letarax-1b-like", 2048, 16, 4, 128, 8192, 8, 1024)
+BUILTIN_SPECS["letarax-8b-like"] = letarax_spec("letarax-8b-like", 4096, 32, 8, 128, 14336, 4, 2048)
+
+
 def _register_test_models():
     # resolvable by name in spawned stage processes too (tests of the multi-process pipeline)
     BUILTIN_SPECS["tiny-llama-test"] = tiny_spec("llama")
@@ -515,6 +533,8 @@ def _register_test_models():
     BUILTIN_SPECS["tiny-qwen2-gpu-test"] = tiny_spec(
         "llama", name="tiny-qwen2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=2, head_dim=64,
         intermediate_size=512, vocab_size=320, num_layers=4, hf_type="qwen2", qkv_bias=True, tie_embeddings=True)
+    BUILTIN_SPECS["tiny-letarax-test"] = letarax_spec("tiny-letarax-test", 64, 4, 2, 16, 96, 4, 12, vocab_size=320, conv=3, pattern="ada")
+    BUILTIN_SPECS["tiny-letarax-gpu-test"] = letarax_spec("tiny-letarax-gpu-test", 128, 4, 2, 64, 256, 4, 40, vocab_size=320)
     BUILTIN_SPECS["tiny-gpt2-gpu-test"] = tiny_spec(
         "gpt2", name="tiny-gpt2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=4, head_dim=64,
         intermediate_size=1024, vocab_size=333, num_layers=4)
