@@ -51,7 +51,6 @@ template <int V> struct IntC { static constexpr int value = V; };
 // clobbers memory (orders the LDS stores) and is followed by a scheduling barrier (orders the
 // MFMAs); (2) the compiler must not COPY a destination between load and wait. A register-tied
 // wait operand provoked exactly such copies in the peeled tail, so the wait names no registers.
-// ops/isa_lint.py re-checks (2) on the generated ISA at build time.
 __device__ __forceinline__ void gload16(u32x4& dst, const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p));
 }
