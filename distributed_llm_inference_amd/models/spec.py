@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import json
 import os
+import math
 from dataclasses import dataclass, asdict, replace
 from typing import Optional, Dict, Any
 
@@ -36,6 +37,15 @@ class RopeScaling:
     truncate: bool = True
 
 
+def distance_bucket(n: int, rows: int, far: int) -> int:
+    """Row of a distance-bias table of `rows` rows for a distance n >= 0: one row per distance below rows / 2,
+    then rows spaced logarithmically up to the distance `far`, the last row for everything beyond."""
+    half = rows // 2
+    if n < half:
+        return n
+    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
+
+
 @dataclass(frozen=True)
 class LayerSpec:
     """One layer of a model whose layers differ from each other (a hybrid stack): which token mixer it
@@ -47,8 +57,21 @@ class LayerSpec:
     value); `scale` multiplies the scores; `rope` says whether positions rotate q and k; `v_mix`: the
     layer's values are blended with those of the first such layer of the stack, by a learned scalar.
     ``delta``: a gated delta-rule recurrence per head over a [dim, vdim] state, q / k shared by
-    `heads // kv_heads` heads, each of q, k, v behind a causal convolution of `conv` taps."""
-    kind: str                       # "attention" | "delta"
+    `heads // kv_heads` heads, each of q, k, v behind a causal convolution of `conv` taps.
+    ``general_delta``: a delta rule with a decay per key channel (from a projection of low rank `rank`) and a
+    removal rate per key channel along the unit key, over a [dim, dim] state per head.
+    ``mlstm``: a matrix memory with exponential input / forget gates (log gates capped at `gate_cap`) kept in
+    range by a running maximum, over a [dim, vdim] state, a [dim] normaliser and the maximum per head.
+    ``parallel``: the mixers in `branches` read the same input; their outputs are RMS-normed over the width
+    and averaged.
+    Further switches of ``attention``: `bias_rows` > 0 adds a learned bias per (distance bucket, head) to the
+    scaled scores (one bucket per distance below bias_rows / 2, logarithmic buckets up to `bias_max`);
+    `head_temp` multiplies a head's scaled scores by a learned number; `sink_learned` makes the sink's score a
+    learned number per head instead of 0; `head_gate` multiplies a head's output by the sigmoid of one more
+    projection of the mixer's input.
+    The feed-forward sublayer is `ff_kind`: ``gated_gelu`` (gelu_tanh(gate) * up, biases), ``gelu`` (up, exact
+    GELU, down; no biases) or ``moe`` (`moe` says how tokens are routed to its experts)."""
+    kind: str                       # "attention" | "delta" | "general_delta" | "mlstm" | "parallel"
     heads: int
     kv_heads: int
     dim: int
@@ -60,21 +83,38 @@ class LayerSpec:
     rope: bool = False
     v_mix: bool = False
     conv: int = 0
+    bias_rows: int = 0
+    bias_max: int = 0
+    head_temp: bool = False
+    sink_learned: bool = False
+    head_gate: bool = False
+    gate_cap: float = 0.0
+    rank: int = 0
+    branches: tuple = ()
+    ff_kind: str = "gated_gelu"
+    moe: Optional["MoeSpec"] = None
 
     @property
     def group(self) -> int:
         return self.heads // self.kv_heads
 
     @property
-    def qk_heads(self) -> int:
-        """Heads of the q projection: every query head for attention, the shared q / k heads for the delta rule."""
-        return self.heads if self.kind == "attention" else self.kv_heads
+    def has_state(self) -> bool:
+        """The mixer keeps a per-sequence state in the sequence's slot."""
+        return self.kind in ("delta", "general_delta", "mlstm") or any(b.has_state for b in self.branches)
 
     @property
-    def v_heads(self) -> int:
-        return self.kv_heads if self.kind == "attention" else self.heads
+    def has_ff(self) -> bool:
+        return self.ff > 0 or self.moe is not None
 
     def mixer_param_count(self, width: int) -> int:
+        if self.kind == "parallel":
+            return sum(b.mixer_param_count(width) + width for b in self.branches)
+        if self.kind == "general_delta":
+            n = self.heads * self.dim
+            return 6 * n * width + 2 * (self.rank or 16) * (width + n) // 2 + 3 * n
+        if self.kind == "mlstm":
+            return width * self.heads * (2 * self.dim + 3 * self.vdim + 2) + 2 * self.heads + self.heads * self.vdim
         qn, kn, vn = self.qk_heads * self.dim, self.kv_heads * self.dim, self.v_heads * self.vdim
         n = width * (qn + kn + vn) + self.heads * self.vdim * width
         if self.kind == "attention":
@@ -82,13 +122,33 @@ class LayerSpec:
         return n + self.conv * (qn + kn + vn) + 2 * self.heads * width + 2 * self.heads + self.vdim + self.heads * self.vdim * width
 
     def ff_param_count(self, width: int) -> int:
+        if self.moe is not None:
+            return self.moe.experts * (3 * width * self.moe.ff + width)
+        if self.ff_kind == "gelu":
+            return 2 * width * self.ff
         return 3 * width * self.ff + 2 * self.ff + width if self.ff else 0
+
+
+@dataclass(frozen=True)
+class MoeSpec:
+    """A routed feed-forward: `experts` small gated feed-forwards of width `ff`, of which a token runs `top`.
+    Scores are the sigmoids of the router's logits. The experts form `groups` equal groups of neighbours; a
+    group's score is the sum of its two largest scores and only experts of the `keep` best groups can be
+    chosen. The chosen scores, divided by their sum and multiplied by `scale`, weigh the experts' outputs. An
+    expert computes down(g sigmoid(1.702 g) (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), +-limit)."""
+    experts: int
+    top: int
+    ff: int
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    limit: float = 7.0
 
 
 @dataclass(frozen=True)
 class ModelSpec:
     name: str
-    family: str                     # "llama" | "gpt2" | "letarax"
+    family: str                     # "llama" | "gpt2" | "letarax" | "nufapel"
     num_layers: int
     hidden_size: int
     num_heads: int
@@ -116,6 +176,16 @@ class ModelSpec:
     # hybrid stacks (family "letarax"): one entry per layer; the scalar fields above then hold the width, the
     # vocabulary and, for the sizes that differ per layer, the largest value over the layers
     layer_specs: tuple = ()
+    # how a hybrid stack wraps its sublayers. "rms": RMS norms before and after every sublayer (weights stored as the
+    # distance from one). "dyt": one dynamic-tanh norm tanh(alpha x) w + b before every sublayer (no statistics), also
+    # as the final norm. `gated_residual`: a sublayer's output is multiplied by sigmoid(W h + b) of the sublayer's input
+    norm_kind: str = "rms"
+    gated_residual: bool = False
+    # (start, stop, times): layers start .. stop-1 run `times` times in a row with the same weights, every pass with a
+    # cache / state of its own and behind a learned vector added to the residual stream
+    loop: tuple = ()
+    learned_positions: bool = False          # a learned vector per position is added to the embedding
+    logit_softcap: float = 0.0               # > 0: logits <- cap tanh(logits / cap)
 
     @property
     def is_hybrid(self) -> bool:
@@ -125,7 +195,19 @@ class ModelSpec:
     def has_recurrent_state(self) -> bool:
         """Some layer keeps a per-sequence state that lives in the sequence's slot (not in cache blocks): a sequence
         cannot change slots without its state being moved along."""
-        return any(l.kind == "delta" for l in self.layer_specs)
+        return any(l.has_state for l in self.layer_specs)
+
+    def layer_runs(self):
+        """[(layer, pass)] in the order the layers run; pass is -1 outside the repeated stretch, else the number of the
+        pass (the stretch's first layer starts a pass). Every run owns a cache / state of its own."""
+        n = len(self.layer_specs)
+        if not self.loop:
+            return [(i, -1) for i in range(n)]
+        start, stop, times = self.loop
+        runs = [(i, -1) for i in range(start)]
+        for t in range(times):
+            runs += [(i, t) for i in range(start, stop)]
+        return runs + [(i, -1) for i in range(stop, n)]
 
     def check_context(self, max_seq_len: int):
         """Attention here is over the whole context. A checkpoint trained with a sliding window gives
@@ -237,6 +319,91 @@ class ModelSpec:
             tie_embeddings=True, bos_token_id=cfg.get("bos_token_id"), eos_token_id=_scalar_eos(cfg.get("eos_token_id")),
             hf_type="letarax", layer_specs=tuple(layers))
 
+    @staticmethod
+    def from_nufapel_config(cfg: Dict[str, Any], name: str = "") -> "ModelSpec":
+        """Nufapel: a hybrid stack listed layer by layer in ``layers``. A layer's ``type`` is ``general_delta`` (mixer:
+        heads, dim) or ``parallel`` (mixer.left: attention with heads, kv_heads, dim, vdim, scale, bias_max, a distance-bias
+        table, head temperatures, learned sinks and head gates; mixer.right: matrix memory with heads, dim, vdim,
+        gate_cap); its ``mlp`` is null, ``dense`` (ff) or ``moe`` (expert.ff, expert.limit, router.experts / top / scale /
+        groups.count / groups.keep). ``loop`` (start, stop, times) repeats a stretch of layers. Dynamic-tanh norms, gated
+        residuals, learned positions (``max_positions``), a head of its own and ``logit_softcap``."""
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m, mlp = l["mixer"], l.get("mlp")
+            ffkw: Dict[str, Any] = dict(ff=0, ff_kind="gelu")
+            if mlp is not None and mlp.get("kind", "dense") == "dense":
+                ffkw = dict(ff=int(mlp["ff"]), ff_kind="gelu")
+            elif mlp is not None and mlp["kind"] == "moe":
+                r, e = mlp["router"], mlp["expert"]
+                g = r.get("groups") or {}
+                moe = MoeSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(e["ff"]), groups=int(g.get("count", 1)),
+                              keep=int(g.get("keep", g.get("count", 1))), scale=float(r.get("scale", 1.0)), limit=float(e["limit"]))
+                if moe.experts % moe.groups or not 1 <= moe.keep <= moe.groups or not 1 <= moe.top <= moe.keep * (moe.experts // moe.groups):
+                    raise ValueError(f"layer {i}: {moe.experts} experts in {moe.groups} groups, {moe.keep} kept, {moe.top} chosen")
+                ffkw = dict(ff=0, ff_kind="moe", moe=moe)
+            elif mlp is not None:
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported (dense and moe are)")
+            if l["type"] == "general_delta":
+                layers.append(LayerSpec("general_delta", heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]),
+                                        vdim=int(m["dim"]), rank=int(m.get("rank", 0)), **ffkw))
+            elif l["type"] == "parallel":
+                a, b = m["left"], m["right"]
+                if int(a["heads"]) % int(a["kv_heads"]):
+                    raise ValueError(f"layer {i}: {a['heads']} heads over {a['kv_heads']} key / value heads")
+                left = LayerSpec("attention", heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                                 scale=float(a["scale"]), sink=True, sink_learned=True, head_temp=True, head_gate=True,
+                                 bias_rows=int(a.get("bias_rows", 0)), bias_max=int(a["bias_max"]))
+                right = LayerSpec("mlstm", heads=int(b["heads"]), kv_heads=int(b["heads"]), dim=int(b["dim"]), vdim=int(b["vdim"]),
+                                  gate_cap=float(b["gate_cap"]), scale=float(b["dim"]) ** -0.5)
+                layers.append(LayerSpec("parallel", heads=left.heads, kv_heads=left.kv_heads, dim=left.dim, vdim=left.vdim,
+                                        branches=(left, right), **ffkw))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        if not layers:
+            raise ValueError("a model needs at least one layer")
+        loop = cfg.get("loop") or None
+        lp = ()
+        if loop and int(loop.get("times", 1)) >= 1 and int(loop["stop"]) > int(loop["start"]):
+            lp = (int(loop["start"]), int(loop["stop"]), int(loop["times"]))
+            if not 0 <= lp[0] < lp[1] <= len(layers):
+                raise ValueError(f"loop {lp} does not fit {len(layers)} layers")
+        heads = [b for l in layers for b in (l.branches or (l,))]
+        return ModelSpec(
+            name=name or "nufapel", family="nufapel", num_layers=len(layers), hidden_size=int(cfg["width"]),
+            num_heads=max(l.heads for l in heads), num_kv_heads=max(l.kv_heads for l in heads),
+            head_dim=max(max(l.dim, l.vdim) for l in heads),
+            intermediate_size=max(max(l.ff, l.moe.ff if l.moe else 0) for l in layers),
+            vocab_size=int(cfg["vocab"]), max_position=int(cfg["max_positions"]), norm_eps=float(cfg["norm"]["eps"]),
+            tie_embeddings=False, bos_token_id=cfg.get("bos_token_id"), eos_token_id=_scalar_eos(cfg.get("eos_token_id")),
+            hf_type="nufapel", layer_specs=tuple(layers), norm_kind="dyt", gated_residual=True, loop=lp,
+            learned_positions=True, logit_softcap=float(cfg.get("logit_softcap") or 0.0))
+
+    def nufapel_config(self) -> Dict[str, Any]:
+        """The inverse of `from_nufapel_config` (`bias_rows` and `rank` are sizes a checkpoint's tensors give; they are
+        written so that random weights of the same shapes can be drawn from the config alone)."""
+        out = []
+        for l in self.layer_specs:
+            if l.kind == "general_delta":
+                m: Dict[str, Any] = {"heads": l.heads, "dim": l.dim, "rank": l.rank}
+            else:
+                a, b = l.branches
+                m = {"left": {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
+                              "bias_max": a.bias_max, "bias_rows": a.bias_rows},
+                     "right": {"heads": b.heads, "dim": b.dim, "vdim": b.vdim, "gate_cap": b.gate_cap}}
+            if l.moe is not None:
+                e = l.moe
+                mlp = {"kind": "moe", "expert": {"ff": e.ff, "limit": e.limit},
+                       "router": {"experts": e.experts, "top": e.top, "scale": e.scale, "groups": {"count": e.groups, "keep": e.keep}}}
+            else:
+                mlp = {"kind": "dense", "ff": l.ff} if l.ff else None
+            out.append({"type": l.kind, "mixer": m, "mlp": mlp})
+        cfg = {"architecture": "Nufapel", "layers": out, "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size,
+               "width": self.hidden_size, "max_positions": self.max_position, "logit_softcap": self.logit_softcap,
+               "bos_token_id": self.bos_token_id, "eos_token_id": self.eos_token_id}
+        if self.loop:
+            cfg["loop"] = {"start": self.loop[0], "stop": self.loop[1], "times": self.loop[2]}
+        return cfg
+
     def letarax_config(self) -> Dict[str, Any]:
         """The inverse of `from_letarax_config`."""
         out = []
@@ -258,6 +425,8 @@ class ModelSpec:
         archs = cfg.get("architectures") or []
         if cfg.get("architecture") == "Letarax":
             return ModelSpec.from_letarax_config(cfg, name=name)
+        if cfg.get("architecture") == "Nufapel":
+            return ModelSpec.from_nufapel_config(cfg, name=name)
         if mt == "gpt2" or any("GPT2" in a for a in archs):
             if cfg.get("activation_function", "gelu_new") != "gelu_new" or cfg.get("scale_attn_by_inverse_layer_idx"):
                 raise ValueError("GPT-2 variants other than gelu_new MLPs with plain 1/sqrt(d) attention scaling are not supported")
@@ -389,7 +558,7 @@ class ModelSpec:
     def hf_config(self) -> Dict[str, Any]:
         """The inverse of `from_hf_config`: a config.json dict for this spec."""
         if self.is_hybrid:
-            return self.letarax_config()
+            return self.nufapel_config() if self.family == "nufapel" else self.letarax_config()
         if self.is_gpt2:
             return {
                 "model_type": "gpt2", "architectures": ["GPT2LMHeadModel"],

@@ -13,6 +13,7 @@ be sampled go through the final norm and lm_head.
 """
 from __future__ import annotations
 
+import math
 from typing import Dict, List, Optional
 
 import torch
@@ -53,7 +54,10 @@ class RefStage:
     def _slot_cache(self, slot: int):
         c = self.cache.get(slot)
         if c is None:
-            if self.spec.is_hybrid:
+            if self.spec.is_hybrid and self.spec.norm_kind == "dyt":
+                # one entry per layer RUN (a repeated stretch of layers owns a cache / state per pass)
+                c = [self._fresh_layer_state(self.spec.layer_specs[i]) for i, _ in self.spec.layer_runs()]
+            elif self.spec.is_hybrid:
                 c = [self._fresh_layer_state(self.spec.layer_specs[i]) for i in self.plan.layers]
             else:
                 z = lambda: torch.zeros(0, self.spec.num_kv_heads, self.spec.head_dim, dtype=self.dtype, device=self.device)
@@ -63,6 +67,13 @@ class RefStage:
 
     def _fresh_layer_state(self, ls):
         dev = self.device
+        z32 = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device=dev)
+        if ls.kind == "parallel":
+            return [self._fresh_layer_state(b) for b in ls.branches]
+        if ls.kind == "general_delta":
+            return [z32(ls.heads, ls.dim, ls.dim)]
+        if ls.kind == "mlstm":
+            return [z32(ls.heads, ls.dim, ls.vdim), z32(ls.heads, ls.dim), z32(ls.heads)]
         if ls.kind == "attention":
             return [torch.zeros(0, ls.kv_heads, ls.dim, dtype=self.dtype, device=dev),
                     torch.zeros(0, ls.kv_heads, ls.vdim, dtype=self.dtype, device=dev)]
@@ -156,10 +167,105 @@ class RefStage:
                 h = h + R.rmsnorm(lin(act, l["w_down"], l["b_down"]), l["ln2b_w"], eps, unit_offset=True)
         return h
 
+    # -- hybrid stacks with dynamic-tanh pre-norms and gated residuals -------------------------------------------
+    def _gated_layers(self, batch: StepBatch, h: torch.Tensor) -> torch.Tensor:
+        """x <- x + sigmoid(W_g n + b_g) * f(n), n = dyt(x), for the mixer and the feed-forward of every layer run. Norms,
+        scores, routers, gates of the recurrences, their states and the residual sum are fp32 whatever the dtype."""
+        spec, dt, eps, w = self.spec, self.dtype, self.spec.norm_eps, self.w
+        T = h.shape[0]
+        F = torch.nn.functional
+        lin = lambda x, m, b=None: R.gemm(x.to(dt), m, b, None, 1 if b is not None else 0)
+        rnd = lambda x: x.to(dt).float()
+        seqs = []
+        t0 = 0
+        for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+            if qlen > 0 and ctx == 0:
+                self.cache.pop(slot, None)            # a sequence's first tokens: whatever the slot held before is void
+            if qlen > 0:
+                seqs.append((slot, t0, qlen, ctx))
+            t0 += qlen
+        self.layer_outputs = []
+        for ri, (li, pas) in enumerate(spec.layer_runs()):
+            ls, l = spec.layer_specs[li], w.layers[li]
+            if pas >= 0 and li == spec.loop[0]:
+                h = h + w.loop_step[pas].float()
+            xn = R.dyt(h, l["ln1_w"], l["ln1_b"], l["ln1_a"])
+            z = lin(xn, l["w_in"])
+            if ls.kind == "general_delta":
+                H, d = ls.heads, ls.dim
+                n = H * d
+                r_, k_, v_, g_, a_, w1 = torch.split(z, [n] * 5 + [z.shape[1] - 5 * n], dim=1)
+                dec = torch.exp(-math.exp(-0.5) * torch.sigmoid(lin(torch.tanh(rnd(w1)), l["w_w2"]) + l["w0"].float()))
+                a_ = torch.sigmoid(a_ + l["b_a"].float())
+                o = torch.empty(T, H, d, dtype=torch.float32, device=self.device)
+                for slot, s0, qlen, ctx in seqs:
+                    st, sl = self._slot_cache(slot)[ri], slice(s0, s0 + qlen)
+                    hv = lambda x: x[sl].reshape(qlen, H, d)
+                    o[sl], st[0] = R.general_delta_rule(hv(r_), hv(k_), hv(v_), hv(dec), hv(a_), st[0])
+                mixed = (R.rmsnorm(o, torch.ones(d, device=self.device), eps).reshape(T, n) * l["o_norm_w"].float() * torch.sigmoid(g_))
+                y = lin(mixed, l["w_o"])
+            else:
+                a, b = ls.branches
+                sizes = [a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, a.heads, b.heads * b.dim, b.heads * b.dim,
+                         b.heads * b.vdim, b.heads * b.vdim, b.heads, b.heads]
+                q, k, v, gl, rq, rk, rv, rg, ri_, rf_ = torch.split(z, sizes, dim=1)
+                bias = R.distance_bias_table(l["rel"], a.bias_max, max(c + n_ for _, _, n_, c in seqs))
+                left = torch.empty(T, a.heads, a.vdim, dtype=torch.float32, device=self.device)
+                right = torch.empty(T, b.heads, b.vdim, dtype=torch.float32, device=self.device)
+                li_ = b.gate_cap * torch.tanh((ri_ + l["b_if"][:b.heads].float()) / b.gate_cap)
+                lf_ = F.logsigmoid(b.gate_cap * torch.tanh((rf_ + l["b_if"][b.heads:].float()) / b.gate_cap))
+                for slot, s0, qlen, ctx in seqs:
+                    sta, stb = self._slot_cache(slot)[ri]
+                    sl = slice(s0, s0 + qlen)
+                    assert sta[0].shape[0] >= ctx, f"slot {slot}: cache has {sta[0].shape[0]} tokens, step says {ctx}"
+                    sta[0] = torch.cat([sta[0][:ctx], k[sl].reshape(qlen, a.kv_heads, a.dim).to(dt)])
+                    sta[1] = torch.cat([sta[1][:ctx], v[sl].reshape(qlen, a.kv_heads, a.vdim).to(dt)])
+                    left[sl] = R.attention(q[sl].reshape(qlen, a.heads, a.dim).to(dt), sta[0], sta[1], ctx, a.scale, sink=True,
+                                           temp=l["temp"], dist_bias=bias, sink_logit=l["sink"])
+                    right[sl], stb[0], stb[1], stb[2] = R.matrix_memory(
+                        rq[sl].reshape(qlen, b.heads, b.dim) * b.scale, rk[sl].reshape(qlen, b.heads, b.dim),
+                        rv[sl].reshape(qlen, b.heads, b.vdim), li_[sl], lf_[sl], stb[0], stb[1], stb[2])
+                left = (left * torch.sigmoid(gl).unsqueeze(2)).reshape(T, -1)
+                right = R.rmsnorm(right, torch.ones(b.vdim, device=self.device), eps).reshape(T, -1) * l["o_norm_w"].float() * torch.sigmoid(rg)
+                y = 0.5 * (R.rmsnorm(lin(left, l["w_o"]), l["out_l"], eps) + R.rmsnorm(lin(right, l["w_o_r"]), l["out_r"], eps))
+            h = h + torch.sigmoid(lin(xn, l["w_rg1"], l["b_rg1"])) * y
+            if ls.has_ff:
+                xn = R.dyt(h, l["ln2_w"], l["ln2_b"], l["ln2_a"])
+                if ls.moe is None:
+                    y = lin(rnd(R.gelu_erf(lin(xn, l["w_up"]))), l["w_down"])
+                else:
+                    e = ls.moe
+                    idx, wts = R.moe_route(torch.sigmoid(lin(xn, l["w_router"])), e.top, e.groups, e.keep, e.scale)
+                    y = torch.zeros_like(h)
+                    for ex in range(e.experts):
+                        rows, col = (idx == ex).nonzero(as_tuple=True)
+                        if rows.numel() == 0:
+                            continue
+                        g = lin(xn[rows], l["w_gate_e"][ex]).clamp(max=e.limit)
+                        u = lin(xn[rows], l["w_up_e"][ex]).clamp(min=-e.limit, max=e.limit)
+                        y.index_add_(0, rows, lin(rnd(g * torch.sigmoid(1.702 * g) * (u + 1.0)), l["w_down_e"][ex]) * wts[rows, col].unsqueeze(1))
+                h = h + torch.sigmoid(lin(xn, l["w_rg2"], l["b_rg2"])) * y
+            self.layer_outputs.append(h)
+        return h
+
     def _forward_hybrid(self, batch: StepBatch, x: torch.Tensor) -> torch.Tensor:
         T = batch.num_tokens
         ids = torch.as_tensor(x).to(self.device).long().reshape(-1)
         assert ids.numel() == T, f"expected {T} token ids, got {ids.numel()}"
+        if self.spec.norm_kind == "dyt":
+            pos = torch.tensor([c + i for c, q in zip(batch.ctx_lens, batch.q_lens) for i in range(q)], dtype=torch.long, device=self.device)
+            h = self.w.embed[ids].float()
+            if self.spec.learned_positions:
+                h = h + self.w.pos_embed[pos].float()
+            h = self._gated_layers(batch, h)
+            self.last_hidden = h
+            rows = self._out_rows(batch)
+            if not rows:
+                return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+            hn = R.dyt(h[rows], self.w.final_norm_w, self.w.final_norm_b, self.w.final_norm_a)
+            z = R.gemm(hn.to(self.dtype), self.w.lm_head).float()
+            cap = self.spec.logit_softcap
+            return cap * torch.tanh(z / cap) if cap > 0 else z
         h = self._hybrid_layers(batch, self.w.embed[ids].float())
         self.last_hidden = h
         rows = self._out_rows(batch)

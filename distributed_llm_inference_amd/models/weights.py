@@ -60,6 +60,8 @@ class StageWeights:
     final_norm_w: Optional[torch.Tensor] = None
     final_norm_b: Optional[torch.Tensor] = None
     lm_head: Optional[torch.Tensor] = None
+    final_norm_a: Optional[torch.Tensor] = None      # dynamic-tanh norms: the scalar inside the tanh
+    loop_step: Optional[torch.Tensor] = None         # [passes, H]: added to the residual stream ahead of each pass of a repeated stretch
 
     def num_bytes(self) -> int:
         seen, total = set(), 0
@@ -72,7 +74,7 @@ class StageWeights:
         return total
 
     def tensors(self):
-        for t in (self.embed, self.pos_embed, self.final_norm_w, self.final_norm_b, self.lm_head):
+        for t in (self.embed, self.pos_embed, self.final_norm_w, self.final_norm_b, self.lm_head, self.final_norm_a, self.loop_step):
             if t is not None:
                 yield t
         for l in self.layers:
@@ -91,6 +93,7 @@ class StageWeights:
         out.layers = [{k: cv(v) for k, v in l.items()} for l in self.layers]
         out.final_norm_w = cv(self.final_norm_w)
         out.final_norm_b = cv(self.final_norm_b)
+        out.final_norm_a, out.loop_step = cv(self.final_norm_a), cv(self.loop_step)
         out.lm_head = out.embed if tied else cv(self.lm_head)
         return out
 
@@ -116,9 +119,138 @@ def _randn(name, shape, seed, device, dtype, std=0.02):
     return t.to(dtype)
 
 
+# ---- Nufapel: checkpoint names <-> the logical layout --------------------------------------------------------------
+# Per layer: ln1_w / ln1_b / ln1_a (and ln2_*) dynamic-tanh norms; w_rg1 / b_rg1 (w_rg2 / b_rg2) residual gates;
+#   general_delta: w_in = r | k | v | g | a | w1 (one GEMM), b_a, w_w2 [heads dim, rank], w0, o_norm_w, w_o
+#   parallel:      w_in = left q | k | v | g, right q | k | v | g | i | f; rel [rows, heads], temp, sink, w_o (left);
+#                  b_if, o_norm_w, w_o_r (right); out_l, out_r (the branches' RMS weights)
+#   dense:         w_up, w_down            moe: w_router [E, H], w_gate_e / w_up_e [E, ff, H], w_down_e [E, H, ff]
+_GD_IN = ("r", "k", "v", "g", "a", "w1")
+_PAR_IN = ("left.q", "left.k", "left.v", "left.g", "right.q", "right.k", "right.v", "right.g", "right.i", "right.f")
+
+
+def _nufapel_layer_names(ls, p: str) -> Dict[str, object]:
+    """logical name -> checkpoint name, or a tuple of names that are concatenated (dim 0) or stacked (experts)."""
+    m, f = p + "mix.", p + "mlp."
+    n: Dict[str, object] = {"ln1_w": p + "norm1", "ln1_b": p + "norm1.b", "ln1_a": p + "norm1.alpha", "w_rg1": p + "rg1", "b_rg1": p + "rg1.b"}
+    if ls.kind == "general_delta":
+        n.update({"w_in": tuple(m + x for x in _GD_IN), "b_a": m + "a.b", "w_w2": m + "w2", "w0": m + "w0", "o_norm_w": m + "norm", "w_o": m + "o"})
+    else:
+        n.update({"w_in": tuple(m + x for x in _PAR_IN), "rel": m + "left.rel", "temp": m + "left.temp", "sink": m + "left.sink",
+                  "w_o": m + "left.o", "b_if": (m + "right.i.b", m + "right.f.b"), "o_norm_w": m + "right.norm", "w_o_r": m + "right.o",
+                  "out_l": m + "left.out", "out_r": m + "right.out"})
+    if ls.has_ff:
+        n.update({"ln2_w": p + "norm2", "ln2_b": p + "norm2.b", "ln2_a": p + "norm2.alpha", "w_rg2": p + "rg2", "b_rg2": p + "rg2.b"})
+        if ls.moe is not None:
+            n["w_router"] = f + "router"
+            for x in ("gate", "up", "down"):
+                n[f"w_{x}_e"] = [f"{f}e{e}.{x}" for e in range(ls.moe.experts)]
+        else:
+            n.update({"w_up": f + "up", "w_down": f + "down"})
+    return n
+
+
+def _load_nufapel_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
+    w = StageWeights(spec, plan)
+    get = lambda name: rd.get(name).to(device=device, dtype=dtype)
+    w.embed, w.pos_embed, w.lm_head = get("embed"), get("pos"), get("head")
+    w.final_norm_w, w.final_norm_b, w.final_norm_a = get("final.norm"), get("final.norm.b"), get("final.norm.alpha").reshape(())
+    if spec.loop:
+        w.loop_step = get("loop.step")
+    for i in plan.layers:
+        l = {}
+        for k, names in _nufapel_layer_names(spec.layer_specs[i], f"l{i}.").items():
+            if isinstance(names, tuple):
+                l[k] = torch.cat([get(x) for x in names], dim=0)
+            elif isinstance(names, list):
+                l[k] = torch.stack([get(x) for x in names], dim=0)
+            else:
+                l[k] = get(names)
+        w.layers.append(l)
+    return w
+
+
+def _nufapel_in_sizes(ls, l) -> List[int]:
+    if ls.kind == "general_delta":
+        n = ls.heads * ls.dim
+        return [n] * 5 + [l["w_w2"].shape[1]]
+    a, b = ls.branches
+    return [a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, a.heads, b.heads * b.dim, b.heads * b.dim, b.heads * b.vdim,
+            b.heads * b.vdim, b.heads, b.heads]
+
+
+def export_nufapel_state_dict(w: StageWeights) -> Dict[str, torch.Tensor]:
+    """Logical -> checkpoint names (tests, `save` of random models)."""
+    spec = w.spec
+    sd = {"embed": w.embed, "pos": w.pos_embed, "head": w.lm_head, "final.norm": w.final_norm_w, "final.norm.b": w.final_norm_b,
+          "final.norm.alpha": w.final_norm_a}
+    if w.loop_step is not None:
+        sd["loop.step"] = w.loop_step
+    for i, l in zip(w.plan.layers, w.layers):
+        ls = spec.layer_specs[i]
+        for k, names in _nufapel_layer_names(ls, f"l{i}.").items():
+            if isinstance(names, tuple):
+                sizes = _nufapel_in_sizes(ls, l) if k == "w_in" else [l[k].shape[0] // len(names)] * len(names)
+                for x, t in zip(names, torch.split(l[k], sizes)):
+                    sd[x] = t
+            elif isinstance(names, list):
+                for x, t in zip(names, l[k]):
+                    sd[x] = t
+            else:
+                sd[names] = l[k]
+    return {k: v.detach().clone().contiguous() for k, v in sd.items()}
+
+
+def _random_nufapel_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
+    """Random weights with which every mechanism matters: projections at 1 / sqrt(fan-in), gates, biases, sinks,
+    temperatures and distance biases of order one, decays spread over their range."""
+    H, V = spec.hidden_size, spec.vocab_size
+    w = StageWeights(spec, plan)
+    rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
+    one = lambda name, shape, std: torch.ones(shape, device=device, dtype=dtype) + rn(name, shape, std)
+    w.embed, w.pos_embed, w.lm_head = rn("embed", (V, H), 1.0), rn("pos", (spec.max_position, H), 0.5), rn("head", (V, H), 2.0 * H ** -0.5)
+    w.final_norm_w, w.final_norm_b = one("final.norm", (H,), 0.1), rn("final.norm.b", (H,), 0.1)
+    w.final_norm_a = torch.tensor(0.6, device=device, dtype=dtype)
+    if spec.loop:
+        w.loop_step = rn("loop.step", (spec.loop[2], H), 0.5)
+    for i in plan.layers:
+        ls, p = spec.layer_specs[i], f"layers.{i}."
+        l: Dict[str, torch.Tensor] = {}
+        for s_ in ("1", "2") if ls.has_ff else ("1",):
+            l[f"ln{s_}_w"], l[f"ln{s_}_b"] = one(p + f"ln{s_}_w", (H,), 0.1), rn(p + f"ln{s_}_b", (H,), 0.1)
+            l[f"ln{s_}_a"] = torch.tensor(0.4 + 0.05 * ((i + int(s_)) % 5), device=device, dtype=dtype)
+            l[f"w_rg{s_}"], l[f"b_rg{s_}"] = rn(p + f"w_rg{s_}", (H, H), H ** -0.5), rn(p + f"b_rg{s_}", (H,), 0.5)
+        if ls.kind == "general_delta":
+            n, R = ls.heads * ls.dim, ls.rank or 16
+            l["w_in"] = torch.cat([rn(p + "w_in", (5 * n, H), H ** -0.5), rn(p + "w_w1", (R, H), H ** -0.5)])
+            l["b_a"], l["w_w2"], l["w0"] = rn(p + "b_a", (n,), 0.5), rn(p + "w_w2", (n, R), 2.0 * R ** -0.5), rn(p + "w0", (n,), 1.5)
+            l["o_norm_w"], l["w_o"] = one(p + "o_norm_w", (n,), 0.1), rn(p + "w_o", (H, n), n ** -0.5)
+        else:
+            a, b = ls.branches
+            rows = a.bias_rows or 16
+            sizes = _nufapel_in_sizes(ls, None)
+            l["w_in"] = rn(p + "w_in", (sum(sizes), H), H ** -0.5)
+            l["rel"], l["temp"], l["sink"] = rn(p + "rel", (rows, a.heads), 1.0), one(p + "temp", (a.heads,), 0.3), rn(p + "sink", (a.heads,), 1.0)
+            l["w_o"] = rn(p + "w_o", (H, a.heads * a.vdim), (a.heads * a.vdim) ** -0.5)
+            l["b_if"] = rn(p + "b_if", (2 * b.heads,), 1.0)
+            l["o_norm_w"], l["w_o_r"] = one(p + "o_norm_w", (b.heads * b.vdim,), 0.1), rn(p + "w_o_r", (H, b.heads * b.vdim), (b.heads * b.vdim) ** -0.5)
+            l["out_l"], l["out_r"] = one(p + "out_l", (H,), 0.1), one(p + "out_r", (H,), 0.1)
+        if ls.moe is not None:
+            e = ls.moe
+            l["w_router"] = rn(p + "w_router", (e.experts, H), 2.0 * H ** -0.5)
+            l["w_gate_e"], l["w_up_e"] = rn(p + "w_gate_e", (e.experts, e.ff, H), 1.5 * H ** -0.5), rn(p + "w_up_e", (e.experts, e.ff, H), 1.5 * H ** -0.5)
+            l["w_down_e"] = rn(p + "w_down_e", (e.experts, H, e.ff), e.ff ** -0.5)
+        elif ls.ff:
+            l["w_up"], l["w_down"] = rn(p + "w_up", (ls.ff, H), H ** -0.5), rn(p + "w_down", (H, ls.ff), ls.ff ** -0.5)
+        w.layers.append(l)
+    return w
+
+
 def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
     """Random weights of a hybrid stack, scaled so that activations stay of order one through any depth
     (projections at 1 / sqrt(fan-in), embedding at one) and every bias, convolution tap and gate matters."""
+    if spec.family == "nufapel":
+        return _random_nufapel_weights(spec, plan, seed, device, dtype)
     H, V = spec.hidden_size, spec.vocab_size
     w = StageWeights(spec, plan)
     rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
@@ -152,6 +284,8 @@ def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, 
 
 
 def _load_hybrid_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
+    if spec.family == "nufapel":
+        return _load_nufapel_weights(rd, spec, plan, device, dtype)
     w = StageWeights(spec, plan)
     get = lambda name: rd.get(name).to(device=device, dtype=dtype)
     if plan.has_embed or plan.has_head:

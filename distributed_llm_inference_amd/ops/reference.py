@@ -48,11 +48,13 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, scale: float,
-              window: int = 0, sink: bool = False, k_pos0: int = 0) -> torch.Tensor:
+              window: int = 0, sink: bool = False, k_pos0: int = 0, temp=None, dist_bias=None, sink_logit=None) -> torch.Tensor:
     """One sequence. q [Tq, Hq, D] are the tokens at absolute positions q_pos0.., k [Tk, Hkv, D] and
     v [Tk, Hkv, Dv] hold positions k_pos0..k_pos0+Tk-1 (reaching at least the last query). Causal, GQA.
     `window` > 0: a query at i sees the keys j with 0 <= i - j < window. `sink`: the softmax's
-    denominator has one more term, exp(0), that carries no value. Returns [Tq, Hq, Dv] fp32."""
+    denominator has one more term, exp(0), that carries no value (`sink_logit` [Hq]: exp(sink_logit) instead).
+    `temp` [Hq] multiplies a head's scaled scores; `dist_bias` [distances, Hq] is added to the scaled score of a
+    key at distance i - j (after `temp`). Returns [Tq, Hq, Dv] fp32."""
     Tq, Hq, D = q.shape
     Tk, Hkv, _ = k.shape
     g = Hq // Hkv
@@ -61,12 +63,17 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, sc
     s = torch.einsum("qhd,khd->hqk", q.float(), kf) * scale
     qpos = torch.arange(Tq, device=q.device).view(-1, 1) + q_pos0
     kpos = torch.arange(Tk, device=q.device).view(1, -1) + k_pos0
+    if temp is not None:
+        s = s * temp.float().view(Hq, 1, 1)
+    if dist_bias is not None:
+        s = s + dist_bias.float()[(qpos - kpos).clamp(min=0)].permute(2, 0, 1)
     hidden = kpos > qpos
     if window and window > 0:
         hidden = hidden | (qpos - kpos >= window)
     s = s.masked_fill(hidden.unsqueeze(0), float("-inf"))
     if sink:
-        s = torch.cat([s, s.new_zeros(Hq, Tq, 1)], dim=-1)
+        last = s.new_zeros(Hq, Tq, 1) if sink_logit is None else sink_logit.float().view(Hq, 1, 1).expand(Hq, Tq, 1)
+        s = torch.cat([s, last], dim=-1)
         p = torch.softmax(s, dim=-1)[..., :-1]
     else:
         p = torch.softmax(s, dim=-1)
@@ -104,3 +111,68 @@ def gated_delta_rule(q, k, v, beta, decay, S):
         S = S + kf[t].unsqueeze(2) * u.unsqueeze(1)
         out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
     return out, S
+
+
+def dyt(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, alpha) -> torch.Tensor:
+    """Dynamic tanh in the place of a norm: tanh(alpha x) w + b, no statistics."""
+    return torch.tanh(x.float() * float(alpha)) * w.float() + b.float()
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    return 0.5 * x * (1.0 + torch.erf(x * (2.0 ** -0.5)))
+
+
+def distance_bias_table(rel: torch.Tensor, far: int, distances: int) -> torch.Tensor:
+    """rel [rows, heads] (a learned bias per distance bucket and head) -> [distances, heads], the bias of every
+    distance 0 .. distances-1 (`spec.distance_bucket` maps a distance to its row)."""
+    from ..models.spec import distance_bucket
+    rows = torch.tensor([distance_bucket(n, rel.shape[0], far) for n in range(distances)], dtype=torch.long, device=rel.device)
+    return rel.float()[rows]
+
+
+def general_delta_rule(r, k, v, w, a, S, eps: float = 1e-6):
+    """Token by token, per head: u = k / sqrt(sum k^2 + eps); S <- diag(w) S - (a u) (u^T S) + k v^T (both terms read
+    the old state); o = S^T r. r, k, v, w, a [T, H, d], S [H, d, d] fp32. Returns (o [T, H, d], S)."""
+    rf, kf, vf, wf, af, S = r.float(), k.float(), v.float(), w.float(), a.float(), S.float().clone()
+    u = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + eps)
+    out = torch.empty_like(vf)
+    for t in range(rf.shape[0]):
+        us = torch.einsum("hd,hdv->hv", u[t], S)
+        S = wf[t].unsqueeze(2) * S - (af[t] * u[t]).unsqueeze(2) * us.unsqueeze(1) + kf[t].unsqueeze(2) * vf[t].unsqueeze(1)
+        out[t] = torch.einsum("hdv,hd->hv", S, rf[t])
+    return out, S
+
+
+def matrix_memory(q, k, v, log_i, log_f, S, n, m):
+    """Token by token, per head: m' = max(log_f + m, log_i); S <- exp(log_f + m - m') S + exp(log_i - m') k v^T; n the
+    same with k alone; o = S^T q / (max(|n . q|, exp(-m')) + 1e-6). q, k [T, H, d], v [T, H, dv], log_i, log_f [T, H],
+    S [H, d, dv], n [H, d], m [H] fp32. Returns (o [T, H, dv], S, n, m)."""
+    qf, kf, vf = q.float(), k.float(), v.float()
+    S, n, m = S.float().clone(), n.float().clone(), m.float().clone()
+    out = torch.empty_like(vf)
+    for t in range(qf.shape[0]):
+        new = torch.maximum(log_f[t].float() + m, log_i[t].float())
+        keep, put = torch.exp(log_f[t].float() + m - new), torch.exp(log_i[t].float() - new)
+        S = keep.view(-1, 1, 1) * S + put.view(-1, 1, 1) * kf[t].unsqueeze(2) * vf[t].unsqueeze(1)
+        n = keep.view(-1, 1) * n + put.view(-1, 1) * kf[t]
+        m = new
+        den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+        out[t] = torch.einsum("hdv,hd->hv", S, qf[t]) / den.view(-1, 1)
+    return out, S, n, m
+
+
+def moe_route(scores: torch.Tensor, top: int, groups: int, keep: int, scale: float):
+    """scores [T, E] fp32 (sigmoids of the router's logits) -> (experts [T, top] int64, weights [T, top] fp32). Experts
+    form `groups` equal groups of neighbours; a group's score is the sum of its two largest scores, only experts of the
+    `keep` best groups can be chosen; the `top` largest of them are, weighted by score / (sum + 1e-20) * scale. Equal
+    scores go to the lower index."""
+    T, E = scores.shape
+    per = E // groups
+    sf = scores.float()
+    gs = sf.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+    order = torch.argsort(gs, dim=-1, descending=True, stable=True)[:, :keep]
+    allowed = torch.zeros(T, groups, dtype=torch.bool, device=scores.device).scatter_(1, order, True)
+    masked = sf.masked_fill(~allowed.repeat_interleave(per, dim=1), -1.0)
+    idx = torch.argsort(masked, dim=-1, descending=True, stable=True)[:, :top]
+    val = sf.gather(1, idx)
+    return idx, val / (val.sum(-1, keepdim=True) + 1e-20) * scale
