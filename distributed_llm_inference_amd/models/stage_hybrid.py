@@ -15,6 +15,17 @@ and what a sequence owns: besides its cache blocks (attention layers), one slot 
 state arrays, indexed by the step descriptor's slot number (the row of the block table). A sequence's first
 tokens (context length 0) start from a zero state inside the kernels, so a slot is reused without clearing.
 
+Stacks with dynamic-tanh pre-norms and gated residuals (`spec.norm_kind == "dyt"`) run the same way through
+`_layers_gated`: per layer RUN (a stretch of layers may repeat with the same weights; every run owns its cache and state)
+
+    h (fp32) -> dyt norm -> ONE input GEMM (all projections of the mixer and the residual gate)
+             -> [ decay GEMM (low rank) -> generalised delta rule -> per-head norm * gate -> o GEMM
+                | cache write -> attention with distance bias / head temperature / learned sink / head gate -> o GEMM
+                  beside   matrix memory (exponential gates) -> per-head norm * gate -> o GEMM ]
+             -> gated residual add (+ mean of the two RMS-normed branches) + the next norm (one kernel)
+             -> [ up GEMM -> gelu -> down GEMM | router -> plan -> the experts' GEMMs over sorted rows -> weighted sum ]
+             -> gated residual add + the next norm
+
 Matrix products take bf16 operands (or fp32: `dtype="fp32"`, everything in true 32-bit) and accumulate in
 fp32; norms, scores, softmax, value mixing, gates, decays and states are fp32 in both modes.
 """
@@ -22,6 +33,7 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass
+from types import SimpleNamespace
 from typing import Dict, List, Optional
 
 import torch
@@ -78,6 +90,10 @@ class HybridGpuStage(GpuStage):
                 raise ValueError(f"layer {i}: head sizes up to 512 are supported")
             if ls.kind == "delta" and not 1 <= ls.conv <= 16:
                 raise ValueError(f"layer {i}: 1 to 16 convolution taps are supported")
+        for i, ls in zip(plan.layers, self.specs):
+            for b in ls.branches or (ls,):
+                if max(b.dim, b.vdim) > 512:
+                    raise ValueError(f"layer {i}: head sizes up to 512 are supported")
         mixers = [ls for ls in self.specs if ls.kind == "attention" and ls.v_mix]
         if len({(ls.kv_heads, ls.vdim) for ls in mixers}) > 1:
             raise ValueError("value mixing needs the same key / value heads and value size in every layer that mixes")
@@ -97,48 +113,60 @@ class HybridGpuStage(GpuStage):
         self.mfma_attn = [mfma_ok and ls.kind == "attention" and ls.dim == ls.vdim and ls.dim in (64, 128) and ls.group <= 16
                           for ls in self.specs]
         self._no_rope = {D: torch.zeros(1, D // 2, device=self.device) for D in (64, 128)}
-        self.embed = mat(weights.embed)
-        self.lm_head = self.embed
-        self.lm_head_p = None
-        self.pos_embed = None
-        self.final_norm_w = f32(weights.final_norm_w)
-        self.vocab_pad = packing.padded_n(spec.vocab_size)
-        self.layers: List[Dict[str, torch.Tensor]] = []
-        for i, ls in enumerate(self.specs):
-            l = weights.layers[i]
-            p: Dict[str, torch.Tensor] = {"ln1_w": f32(l["ln1_w"]), "ln1b_w": f32(l["ln1b_w"])}
-            self._matrix(p, "w_o", mat(l["w_o"]), None)
-            if ls.kind == "attention":
-                self._matrix(p, "w_qkv", mat(l["w_qkv"]), f32(l["b_qkv"]))
-                p["vmix"] = f32(l["vmix"]).reshape(1)
-            else:
-                self._matrix(p, "w_in", mat(l["w_in"]), None)
-                p["conv_w"] = f32(l["conv_w"])
-                p["A_log"], p["dt_bias"], p["o_norm_w"] = f32(l["A_log"]), f32(l["dt_bias"]), f32(l["o_norm_w"])
-            if ls.ff:
-                # gate and up rows interleaved in 16-row tiles, so that one wave holds both for the same output
-                # columns; a width that is no multiple of 16 is padded with zero rows (their activations are zero
-                # and meet zero columns of the down projection)
-                pad = (-ls.ff) % 16
-                padr = lambda t: torch.cat([t, t.new_zeros(pad, *t.shape[1:])]) if pad else t
-                p["ln2_w"], p["ln2b_w"] = f32(l["ln2_w"]), f32(l["ln2b_w"])
-                if self._packed and spec.hidden_size % 128 == 0 and ls.ff % 8 == 0:
-                    # gate rows, then up rows, through the packed-weight GEMM; the gate is applied by a kernel of its own
-                    self._matrix(p, "w_gu", torch.cat([mat(l["w_gate"]), mat(l["w_up"])]), torch.cat([f32(l["b_gate"]), f32(l["b_up"])]))
-                    p["ff_cols"] = ls.ff
+        if spec.norm_kind == "dyt":
+            # one cache / state per layer RUN; the attention of these stacks (distance bias, temperatures, learned sinks, head
+            # gates) runs on the any-size kernel
+            self._attn_of_run = [spec.layer_specs[li].branches[0] if spec.layer_specs[li].kind == "parallel" else None for li, _ in spec.layer_runs()]
+            self.mfma_attn = [False] * len(self._attn_of_run)
+        else:
+            self._attn_of_run = [ls if ls.kind == "attention" else None for ls in self.specs]
+        self.gated = spec.norm_kind == "dyt"
+        self.runs = spec.layer_runs()
+        if self.gated:
+            self._load_gated(weights, f32, mat)
+        else:
+            self.embed = mat(weights.embed)
+            self.lm_head = self.embed
+            self.lm_head_p = None
+            self.pos_embed = None
+            self.final_norm_w = f32(weights.final_norm_w)
+            self.vocab_pad = packing.padded_n(spec.vocab_size)
+            self.layers: List[Dict[str, torch.Tensor]] = []
+            for i, ls in enumerate(self.specs):
+                l = weights.layers[i]
+                p: Dict[str, torch.Tensor] = {"ln1_w": f32(l["ln1_w"]), "ln1b_w": f32(l["ln1b_w"])}
+                self._matrix(p, "w_o", mat(l["w_o"]), None)
+                if ls.kind == "attention":
+                    self._matrix(p, "w_qkv", mat(l["w_qkv"]), f32(l["b_qkv"]))
+                    p["vmix"] = f32(l["vmix"]).reshape(1)
                 else:
-                    p["w_gu"] = packing.interleave_gate_up(padr(mat(l["w_gate"])), padr(mat(l["w_up"]))).contiguous()
-                    p["b_gu"] = packing.interleave_gate_up(padr(f32(l["b_gate"])).unsqueeze(1), padr(f32(l["b_up"])).unsqueeze(1)).reshape(-1).contiguous()
-                    p["ff_cols"] = ls.ff + pad
-                wd = mat(l["w_down"])
-                if "w_gu_p" not in p and pad:
-                    wd = torch.cat([wd, wd.new_zeros(wd.shape[0], pad)], dim=1).contiguous()
-                self._matrix(p, "w_down", wd, f32(l["b_down"]))
-            self.layers.append(p)
-            weights.layers[i] = {}
-        if self._packed and spec.hidden_size % 128 == 0:
-            self.lm_head_p = packing.pack_weight(self.embed)
-            self._shapes.append((self.vocab_pad, spec.hidden_size, False))
+                    self._matrix(p, "w_in", mat(l["w_in"]), None)
+                    p["conv_w"] = f32(l["conv_w"])
+                    p["A_log"], p["dt_bias"], p["o_norm_w"] = f32(l["A_log"]), f32(l["dt_bias"]), f32(l["o_norm_w"])
+                if ls.ff:
+                    # gate and up rows interleaved in 16-row tiles, so that one wave holds both for the same output
+                    # columns; a width that is no multiple of 16 is padded with zero rows (their activations are zero
+                    # and meet zero columns of the down projection)
+                    pad = (-ls.ff) % 16
+                    padr = lambda t: torch.cat([t, t.new_zeros(pad, *t.shape[1:])]) if pad else t
+                    p["ln2_w"], p["ln2b_w"] = f32(l["ln2_w"]), f32(l["ln2b_w"])
+                    if self._packed and spec.hidden_size % 128 == 0 and ls.ff % 8 == 0:
+                        # gate rows, then up rows, through the packed-weight GEMM; the gate is applied by a kernel of its own
+                        self._matrix(p, "w_gu", torch.cat([mat(l["w_gate"]), mat(l["w_up"])]), torch.cat([f32(l["b_gate"]), f32(l["b_up"])]))
+                        p["ff_cols"] = ls.ff
+                    else:
+                        p["w_gu"] = packing.interleave_gate_up(padr(mat(l["w_gate"])), padr(mat(l["w_up"]))).contiguous()
+                        p["b_gu"] = packing.interleave_gate_up(padr(f32(l["b_gate"])).unsqueeze(1), padr(f32(l["b_up"])).unsqueeze(1)).reshape(-1).contiguous()
+                        p["ff_cols"] = ls.ff + pad
+                    wd = mat(l["w_down"])
+                    if "w_gu_p" not in p and pad:
+                        wd = torch.cat([wd, wd.new_zeros(wd.shape[0], pad)], dim=1).contiguous()
+                    self._matrix(p, "w_down", wd, f32(l["b_down"]))
+                self.layers.append(p)
+                weights.layers[i] = {}
+            if self._packed and spec.hidden_size % 128 == 0:
+                self.lm_head_p = packing.pack_weight(self.embed)
+                self._shapes.append((self.vocab_pad, spec.hidden_size, False))
         self._ws_floats = self._packed_ws_floats()
         self.keep_layer_outputs = False          # debugging aid: eager steps append the residual stream after every layer
         self.layer_outputs: List[torch.Tensor] = []
@@ -146,7 +174,14 @@ class HybridGpuStage(GpuStage):
         self._init_step_state(kv_mem_fraction, decode_states)
         # recurrent state, one slot per row of the block table (the null slot included: padding rows land there)
         self.rec: List[Optional[tuple]] = []
-        for ls in self.specs:
+        for ls in ([spec.layer_specs[li] for li, _ in self.runs] if self.gated else []):
+            if ls.kind == "general_delta":
+                self.rec.append((torch.zeros(max_slots + 1, ls.heads, ls.dim, ls.dim, device=dev),))
+            else:
+                b = ls.branches[1]
+                self.rec.append((torch.zeros(max_slots + 1, b.heads, b.dim, b.vdim + 1, device=dev),
+                                 torch.zeros(max_slots + 1, b.heads, 128, device=dev)))
+        for ls in ([] if self.gated else self.specs):
             if ls.kind == "delta":
                 C = 2 * ls.kv_heads * ls.dim + ls.heads * ls.vdim
                 self.rec.append((torch.zeros(max_slots + 1, max(ls.conv - 1, 1), C, device=dev),
@@ -200,7 +235,9 @@ class HybridGpuStage(GpuStage):
         return need
 
     # ---- workspaces ---------------------------------------------------------------------------------------
-    def _new_work(self, rows: int) -> _HybridWork:
+    def _new_work(self, rows: int):
+        if self.gated:
+            return self._new_work_gated(rows)
         s, dev, at = self.spec, self.device, self.act_dtype
         z = lambda n, dt=torch.float32: torch.zeros(max(int(n), 1), device=dev, dtype=dt)
         B = min(rows, self.max_batch)
@@ -230,10 +267,13 @@ class HybridGpuStage(GpuStage):
     # ---- cache and state sizing -------------------------------------------------------------------------
     def kv_block_bytes(self) -> int:
         e = 4 if self.act_dtype == torch.float32 else 2
-        return max(1, sum(ls.kv_heads * BLOCK * (ls.dim + ls.vdim) * e for ls in self.specs if ls.kind == "attention"))
+        return max(1, sum(ls.kv_heads * BLOCK * (ls.dim + ls.vdim) * e for ls in self._attn_of_run if ls is not None))
 
     def _decode_state_bytes(self) -> int:
         n = 0
+        if self.gated:
+            per_row = sum(t.numel() * t.element_size() for t in vars(self.wk0).values() if torch.is_tensor(t)) // self.max_tokens
+            return sum(B * (per_row + 4 * self.vocab_pad) for B in self.graph_sizes)
         for B in self.graph_sizes:
             w = self.wk0
             per_row = sum(t.numel() * t.element_size() for t in (w.h, w.xn, w.z, w.y, w.o, w.mixed, w.yo, w.act, w.vfirst)) // self.max_tokens
@@ -245,11 +285,11 @@ class HybridGpuStage(GpuStage):
         self.num_blocks = int(num_blocks)
         # zero-filled: a row that was never written must hold finite values
         # (a layer on the MFMA attention kernels keeps K and V slabs of a block side by side, in fragment order)
-        self.kv = [None if ls.kind != "attention" else
+        self.kv = [None if ls is None else
                    torch.zeros(self.num_blocks, ls.kv_heads, 2, BLOCK * ls.dim, device=dev, dtype=at) if fast else
                    (torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, ls.dim, device=dev, dtype=at),
                     torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, ls.vdim, device=dev, dtype=at))
-                   for ls, fast in zip(self.specs, self.mfma_attn)]
+                   for ls, fast in zip(self._attn_of_run, self.mfma_attn)]
 
     def _pick_splits(self, B: int, max_ctx: int) -> int:
         return 1
@@ -268,10 +308,15 @@ class HybridGpuStage(GpuStage):
 
     # ---- the layer stack ----------------------------------------------------------------------------------
     def _embed_rows(self, wk, T: int, ids, pos):
-        self.K.embed32(wk.h[:T], ids, self.embed)
+        if self.pos_embed is not None:
+            self.K.embed_pos32(wk.h[:T], ids, pos, self.embed, self.pos_embed)
+        else:
+            self.K.embed32(wk.h[:T], ids, self.embed)
 
     def _layers(self, wk: _HybridWork, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int, splits: int,
                 alone: bool = False, lead_decode: int = 0):
+        if self.gated:
+            return self._layers_gated(wk, T, tok_pos, tok_seq, q_start, ctx, slots)
         K, eps = self.K, self.spec.norm_eps
         h, xn, yo = wk.h[:T], wk.xn[:T], wk.yo[:T]
         view = lambda buf, cols: buf[:T * cols].view(T, cols)
@@ -344,24 +389,194 @@ class HybridGpuStage(GpuStage):
                 self.layer_outputs.append(h.clone())
         return None
 
+    # ---- stacks with dynamic-tanh norms and gated residuals -------------------------------------------------------
+    def _load_gated(self, weights: StageWeights, f32, mat):
+        """Device weights of a gated stack. Everything that reads a sublayer's input is ONE matrix: the mixer's projections and
+        the residual gate (mixer), the up projection or the router and the residual gate (feed-forward). Biases stay apart and
+        are added in fp32 by the kernels that consume the projections."""
+        from ..ops import reference as R
+        spec, dev = self.spec, self.device
+        self.embed, self.pos_embed = mat(weights.embed), mat(weights.pos_embed) if spec.learned_positions else None
+        self.lm_head = mat(weights.lm_head)
+        self.lm_head_p = None
+        self.final_norm_w, self.final_norm_b = f32(weights.final_norm_w), f32(weights.final_norm_b)
+        self.final_norm_a = float(weights.final_norm_a)
+        self.loop_step = f32(weights.loop_step) if spec.loop else None
+        self.vocab_pad = packing.padded_n(spec.vocab_size)
+        self.layers = []
+        for i, ls in enumerate(self.specs):
+            l = weights.layers[i]
+            p = {k: f32(l[k]) for k in ("ln1_w", "ln1_b", "b_rg1", "o_norm_w")}
+            p["ln1_a"] = float(l["ln1_a"])
+            self._matrix(p, "w_in", torch.cat([mat(l["w_in"]), mat(l["w_rg1"])]), None)
+            self._matrix(p, "w_o", mat(l["w_o"]), None)
+            if ls.kind == "general_delta":
+                p["rank"] = int(l["w_w2"].shape[1])
+                p["b_a"], p["w0"] = f32(l["b_a"]), f32(l["w0"])
+                self._matrix(p, "w_w2", mat(l["w_w2"]), None)
+            else:
+                a = ls.branches[0]
+                p["bias"] = R.distance_bias_table(l["rel"].float().cpu(), a.bias_max, self.max_seq_len).to(dev).contiguous()
+                for k in ("temp", "sink", "b_if", "out_l", "out_r"):
+                    p[k] = f32(l[k])
+                self._matrix(p, "w_o_r", mat(l["w_o_r"]), None)
+            if ls.has_ff:
+                p.update({k: f32(l[k]) for k in ("ln2_w", "ln2_b", "b_rg2")})
+                p["ln2_a"] = float(l["ln2_a"])
+                if ls.moe is not None:
+                    if ls.moe.experts > 256:
+                        raise ValueError("up to 256 experts are supported")
+                    self._matrix(p, "w_ff", torch.cat([mat(l["w_router"]), mat(l["w_rg2"])]), None)
+                    p["w_gate_e"], p["w_up_e"], p["w_down_e"] = (mat(l[k]) for k in ("w_gate_e", "w_up_e", "w_down_e"))
+                else:
+                    self._matrix(p, "w_ff", torch.cat([mat(l["w_up"]), mat(l["w_rg2"])]), None)
+                    self._matrix(p, "w_down", mat(l["w_down"]), None)
+            self.layers.append(p)
+            weights.layers[i] = {}
+        if self._packed and spec.hidden_size % 128 == 0:
+            self.lm_head_p = packing.pack_weight(self.lm_head)
+            self._shapes.append((self.vocab_pad, spec.hidden_size, False))
+
+    def _new_work_gated(self, rows: int):
+        s, dev, at = self.spec, self.device, self.act_dtype
+        z = lambda n, dt=torch.float32: torch.zeros(max(int(n), 1), device=dev, dtype=dt)
+        B, H = min(rows, self.max_batch), s.hidden_size
+        zc = wc = lc = oc = mc = m2 = z2 = ac = yc = 1
+        pairs = tiles = ef = 0
+        for ls, p in zip(self.specs, self.layers):
+            zc, yc = max(zc, self._cols(p, "w_in")), max(yc, self._cols(p, "w_o"))
+            if ls.kind == "general_delta":
+                n = ls.heads * ls.dim
+                wc, lc, oc, mc = max(wc, self._cols(p, "w_w2")), max(lc, p["rank"]), max(oc, n), max(mc, n)
+            else:
+                a, b = ls.branches
+                mc, m2, oc = max(mc, a.heads * a.vdim), max(m2, b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
+                yc = max(yc, self._cols(p, "w_o_r"))
+            if ls.has_ff:
+                z2 = max(z2, self._cols(p, "w_ff"))
+                if ls.moe is not None:
+                    e = ls.moe
+                    pairs, tiles, ef = max(pairs, rows * e.top), max(tiles, (rows * e.top + 15) // 16 + e.experts), max(ef, e.ff)
+                else:
+                    ac, yc = max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
+        ws_floats = self._ws_floats
+        if self._packed and rows > self.decode_rows:
+            for m_ in {rows, min(rows, 512), min(rows, 1024)}:
+                if m_ > self.decode_rows:
+                    ws_floats = max([ws_floats] + [int(self.K.gemm_ws_floats(m_, n_, k_)) for n_, k_, _ in self._shapes])
+        i32 = torch.int32
+        return SimpleNamespace(
+            h=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), wz=z(rows * wc),
+            low=z(rows * lc, at), o=z(rows * oc), mixed=z(rows * mc, at), mixed2=z(rows * m2, at), ya=z(rows * yc), yb=z(rows * yc),
+            z2=z(rows * z2), act=z(rows * ac, at), sel=z(pairs, i32), wts=z(pairs), pair_row=z(pairs, i32), tiles=z(1 + tiles, i32),
+            row_tok=z(16 * tiles, i32), eact=z(16 * tiles * ef, at), ey=z(16 * tiles * H), ws=z(ws_floats + 4096),
+            head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
+
+    def _layers_gated(self, wk, T: int, tok_pos, tok_seq, q_start, ctx, slots):
+        K, eps, H = self.K, self.spec.norm_eps, self.spec.hidden_size
+        h, xn = wk.h[:T], wk.xn[:T]
+        view = lambda buf, cols: buf[:T * cols].view(T, cols)
+        keep = self.keep_layer_outputs and not torch.cuda.is_current_stream_capturing()
+        if keep:
+            self.layer_outputs = []
+        runs, first = self.runs, (self.spec.loop[0] if self.spec.loop else -1)
+
+        def opening(ri):
+            """(step vector, norm weight, bias, alpha) of what follows run ri - 1: the vector that opens a pass and the first norm of run ri."""
+            if ri >= len(runs):
+                return None, None, None, 0.0
+            li, pas = runs[ri]
+            p = self.layers[li]
+            return (self.loop_step[pas] if pas >= 0 and li == first else None), p["ln1_w"], p["ln1_b"], p["ln1_a"]
+
+        step, nw, nb, na = opening(0)
+        K.dyt_gate(xn, h, None, None, None, None, None, None, step, nw, nb, None, na, eps)
+        for ri, (li, _) in enumerate(runs):
+            ls, p = self.specs[li], self.layers[li]
+            z = view(wk.z, self._cols(p, "w_in"))
+            self._mm(wk, z, xn, p, "w_in")
+            ya, yb = view(wk.ya, self._cols(p, "w_o")), None
+            if ls.kind == "general_delta":
+                n, d, R = ls.heads * ls.dim, ls.dim, p["rank"]
+                low, wz, o, mixed = view(wk.low, R), view(wk.wz, self._cols(p, "w_w2")), view(wk.o, n), view(wk.mixed, n)
+                K.unary_act(low, z[:, 5 * n:5 * n + R], 1)
+                self._mm(wk, wz, low, p, "w_w2")
+                K.state_scan(0, o, z, wz[:, :n], self.rec[ri][0], None, p["b_a"], p["w0"], q_start, ctx, slots, ls.heads, d, d,
+                             0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0)
+                K.headnorm_gate(mixed, o, z[:, 3 * n:4 * n], p["o_norm_w"], ls.heads, d, 0, eps)
+                self._mm(wk, ya, mixed, p, "w_o")
+                g0, wa, wb = 5 * n + R, None, None
+            else:
+                a, b = ls.branches
+                qn, kn, vn, bn, bv = a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, b.heads * b.dim, b.heads * b.vdim
+                c_g = qn + kn + vn
+                c_q = c_g + a.heads
+                c_k, c_v, c_rg, c_i = c_q + bn, c_q + 2 * bn, c_q + 2 * bn + bv, c_q + 2 * bn + 2 * bv
+                kc, vc = self.kv[ri]
+                mixed, mixed2, o = view(wk.mixed, a.heads * a.vdim), view(wk.mixed2, bv), view(wk.o, b.heads * (b.vdim + 2))
+                K.kv_store(z[:, :c_g], None, None, 0, kc, vc, tok_pos, tok_seq, self.block_table, a.kv_heads, a.dim, a.vdim, qn)
+                K.biased_attention(mixed, z, kc, vc, tok_pos, tok_seq, self.block_table, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
+                                   p["temp"], p["bias"], p["sink"], z[:, c_g:c_q])
+                self._mm(wk, ya, mixed, p, "w_o")
+                K.state_scan(1, o, z, None, self.rec[ri][0], self.rec[ri][1], p["b_if"], None, q_start, ctx, slots, b.heads, b.dim, b.vdim,
+                             c_q, c_k, c_v, 0, c_i, c_i + b.heads, b.gate_cap, b.scale)
+                K.headnorm_gate(mixed2, o, z[:, c_rg:c_rg + bv], p["o_norm_w"], b.heads, b.vdim, 2, eps)
+                yb = view(wk.yb, self._cols(p, "w_o"))
+                self._mm(wk, yb, mixed2, p, "w_o_r")
+                g0, wa, wb, yb = c_i + 2 * b.heads, p["out_l"], p["out_r"], yb[:, :H]
+            if ls.has_ff:
+                step, nw, nb, na = None, p["ln2_w"], p["ln2_b"], p["ln2_a"]
+            else:
+                step, nw, nb, na = opening(ri + 1)
+            K.dyt_gate(xn if nw is not None else None, h, ya[:, :H], yb, wa, wb, z[:, g0:g0 + H], p["b_rg1"], step, nw, nb, None, na, eps)
+            if ls.has_ff:
+                z2 = view(wk.z2, self._cols(p, "w_ff"))
+                self._mm(wk, z2, xn, p, "w_ff")
+                if ls.moe is None:
+                    act, ya = view(wk.act, ls.ff), view(wk.ya, self._cols(p, "w_down"))
+                    K.unary_act(act, z2[:, :ls.ff], 0)
+                    self._mm(wk, ya, act, p, "w_down")
+                    g0 = ls.ff
+                else:
+                    e = ls.moe
+                    nt = (T * e.top + 15) // 16 + e.experts
+                    eact, ey, ya = wk.eact[:16 * nt * e.ff].view(16 * nt, e.ff), wk.ey[:16 * nt * H].view(16 * nt, H), view(wk.ya, H)
+                    K.moe_route(wk.sel, wk.wts, z2[:, :e.experts], e.top, e.groups, e.keep, e.scale)
+                    K.moe_plan(wk.tiles, wk.row_tok, wk.pair_row, wk.sel, T * e.top, e.top, e.experts)
+                    K.moe_up(eact, xn, p["w_gate_e"], p["w_up_e"], wk.tiles, wk.row_tok, nt, e.limit)
+                    K.moe_down(ey, eact, p["w_down_e"], wk.tiles, wk.row_tok, nt)
+                    K.moe_combine(ya, ey, wk.pair_row, wk.wts, e.top)
+                    g0 = e.experts
+                step, nw, nb, na = opening(ri + 1)
+                K.dyt_gate(xn if nw is not None else None, h, ya[:, :H], None, None, None, z2[:, g0:g0 + H], p["b_rg2"], step, nw, nb, None, na, eps)
+            if keep:
+                self.layer_outputs.append(h.clone())
+        return None
+
     def _fold(self, wk, T: int, pend):
         return None
 
-    def _head(self, wk: _HybridWork, rows_idx: torch.Tensor, R: int, T: int, pend):
+    def _head(self, wk, rows_idx: torch.Tensor, R: int, T: int, pend):
         K = self.K
         hx = wk.head_x[:R]
-        K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 1.0)
+        if self.gated:
+            K.dyt_gate(hx, wk.h[:T], None, None, None, None, None, None, None, self.final_norm_w, self.final_norm_b, rows_idx[:R],
+                       self.final_norm_a, self.spec.norm_eps)
+        else:
+            K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 1.0)
         if self.lm_head_p is not None:
             K.gemm(wk.logits[:R], hx, self.lm_head_p, None, None, wk.ws, self.vocab_pad, 0, 0, 0)
         else:
             K.gemm_any(wk.logits[:R, :self.spec.vocab_size], hx, self.lm_head, None, 0)
+        if self.spec.logit_softcap > 0:
+            K.softcap(wk.logits[:R], self.spec.vocab_size, self.spec.logit_softcap)
         return wk.logits[:R]
 
     def memory_report(self) -> Dict[str, float]:
         gib = 1 << 30
         size = lambda t: t.numel() * t.element_size()
-        wbytes = size(self.embed) + sum(size(t) for l in self.layers for t in l.values())
+        wbytes = size(self.embed) + sum(size(t) for l in self.layers for t in l.values() if torch.is_tensor(t))
         kvb = sum(sum(size(t) for t in (kv if isinstance(kv, tuple) else (kv,))) for kv in (self.kv or []) if kv is not None)
-        rec = sum(size(c) + size(s) for r in self.rec if r is not None for c, s in [r])
+        rec = sum(size(t) for r in self.rec if r is not None for t in r)
         return {"weights_gib": wbytes / gib, "kv_gib": kvb / gib, "state_gib": rec / gib, "kv_blocks": self.num_blocks,
                 "kv_tokens": self.num_blocks * BLOCK}

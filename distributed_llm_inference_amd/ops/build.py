@@ -54,9 +54,10 @@ def build(verbose: bool = True, force: bool = False, comm: bool = True) -> str:
     tinc = []
     for p in ce.include_paths("cuda"):
         tinc += ["-isystem", p]
-    bsrc, bobj = os.path.join(CSRC, "bindings.cpp"), os.path.join(OBJ, "bindings.o")
-    objs.append(bobj)
-    if force or _stale(bsrc, bobj, headers):
+    for bname in sorted(f for f in os.listdir(CSRC) if f.startswith("bindings") and f.endswith(".cpp")):
+      bsrc, bobj = os.path.join(CSRC, bname), os.path.join(OBJ, bname[:-4] + ".o")
+      objs.append(bobj)
+      if force or _stale(bsrc, bobj, headers):
         jobs.append([hipcc, "-O2", "-std=c++17", "-fPIC", "-x", "c++", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
                      "-DHIPBLAS_V2", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
                      "-Wno-deprecated-declarations", *tinc, "-c", bsrc, "-o", bobj])

@@ -790,7 +790,8 @@ void window_attention(Tensor out, const Tensor& qkv, const Tensor& kcache, const
   dlia_window_attention(out.data_ptr(), qkv.data_ptr<float>(), kcache.data_ptr(), vcache.data_ptr(), is_f32(kcache),
                         tok_pos.data_ptr<int>(), tok_seq.data_ptr<int>(), block_table.data_ptr<int>(), (int)T,
                         (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0), (int)H, (int)G, (int)d, (int)dv,
-                        qkv.stride(0), out.stride(0), (float)scale, (int)window, sink ? 1 : 0, cur_stream());
+                        qkv.stride(0), out.stride(0), (float)scale, (int)window, sink ? 1 : 0, nullptr, nullptr, 0, nullptr, nullptr, 0,
+                        cur_stream());
 }
 
 void short_conv(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, const Tensor& q_start, const Tensor& ctx,

@@ -125,6 +125,7 @@ void dlia_kv_store(const float* qkv, float* vfirst, const float* lam, int mix, v
 void dlia_window_attention(void* out, const float* qkv, const void* kcache, const void* vcache, int f32, const int* tok_pos,
                            const int* tok_seq, const int* block_table, int T, int max_blocks, int num_blocks, int table_rows,
                            int H, int G, int d, int dv, long ldq, long ldo, float scale, int window, int sink,
+                           const float* temp, const float* bias, int bias_rows, const float* sinkv, const float* gate, long ldg,
                            hipStream_t stream);
 
 // v <- (1 - lam) v + lam v_first on the v columns of a bf16 fused qkv activation (mix 2), or v_first <- v (mix 1)
@@ -137,6 +138,36 @@ void dlia_unit_heads(float* x, int T, int heads, int d, long ld, int scaled_head
 int dlia_delta_rule(float* o, const float* y, const float* z, float* state, const float* A_log, const float* dt_bias,
                     const int* q_start, const int* ctx, const int* slots, int B, int G, int Hv, int d, int dv, int C, long ldz,
                     int col_beta, int col_a, int state_rows, int max_q, hipStream_t stream);
+
+// ---- gated_ops.hip --------------------------------------------------------------------------
+void dlia_embed_pos32(float* out, const int* ids, const int* pos, const void* table, const void* ptable, int f32, int T, int H,
+                      int vocab, int max_pos, hipStream_t stream);
+void dlia_dyt_gate(void* out, int out_f32, float* x, const float* ya, const float* yb, const float* wa, const float* wb,
+                   const float* gl, const float* gb, const float* step, const float* nw, const float* nb, const int* row_idx,
+                   int rows, int H, long ldx, long ldy, long ldg, long ldo, float alpha, float eps, hipStream_t stream);
+void dlia_headnorm_gate(void* out, int out_f32, const float* o, const float* gate, const float* w, int T, int heads, int dv,
+                        int extra, long ldo_in, long ldg, long ld_out, float eps, hipStream_t stream);
+void dlia_unary_act(void* act, int out_f32, const float* z, int M, int F, long ldz, long lda, int kind, hipStream_t stream);
+void dlia_softcap(float* z, int M, int V, long ld, float cap, hipStream_t stream);
+
+// ---- state_scan.hip -------------------------------------------------------------------------
+int dlia_state_scan_blocks(int d, int ncols);
+int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, const float* wz, long ldw, float* state, float* mstate,
+                    const float* b0, const float* b1, const int* q_start, const int* ctx, const int* slots, int B, int H, int d,
+                    int dv, int state_rows, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap,
+                    float qscale, hipStream_t stream);
+
+// ---- moe.hip --------------------------------------------------------------------------------
+void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, int E, int top, int groups, int keep, float scale,
+                    hipStream_t stream);
+void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows,
+                   hipStream_t stream);
+void dlia_moe_up(void* act, const void* x, const void* wg, const void* wu, int f32, const int* tiles, const int* row_tok,
+                 int max_tiles, int F, int K, long ldx, long lda, float limit, hipStream_t stream);
+void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok, int max_tiles, int H,
+                   int F, long lda, hipStream_t stream);
+void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
+                      hipStream_t stream);
 
 // ---- misc.hip -------------------------------------------------------------------------
 void dlia_advance_i32(int* x, int n, int delta, hipStream_t stream);

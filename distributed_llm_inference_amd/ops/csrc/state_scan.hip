@@ -1,0 +1,203 @@
+// Linear recurrences over a per-sequence matrix state, token by token, everything in fp32. One kernel, two rules:
+//
+//   rule 0, generalised delta rule, state S [d, d] per head:
+//       u = k / sqrt(sum k^2 + 1e-6);  S <- diag(w) S - (a u) (u^T S) + k v^T  (both terms read the old S);  o = S^T r
+//       w = exp(-exp(-1/2) sigmoid(wz + w0)),  a = sigmoid(za + ba)   (a decay and a removal rate per key channel)
+//   rule 1, matrix memory with exponential gates, state S [d, dv], normaliser n [d], running maximum m per head:
+//       i = cap tanh((zi + bi) / cap),  f = logsigmoid(cap tanh((zf + bf) / cap)),  m' = max(f + m, i)
+//       S <- exp(f + m - m') S + exp(i - m') k v^T,  n the same with k alone;  the kernel writes the raw read-out S^T q,
+//       n . q and exp(-m') per head ([dv | n.q | exp(-m')] per head in `o`); the division by max(|n . q|, exp(-m')) + 1e-6
+//       happens where the read-out is normalised per head. n is kept as one more column of the state (its "value" is 1).
+//
+// Both rules act on every column of the state alone, so the work is split by columns: a workgroup owns (sequence, head,
+// a block of CB columns), a column's d rows live in the registers of R neighbouring lanes (16 rows each, rows beyond d are
+// zero), the dot products over d are finished with R-lane shuffles. The step's tokens go through LDS in chunks: all threads
+// load a chunk's per-token vectors and evaluate the gates (a token per 16 lanes), then every lane walks the chunk's tokens
+// over its registers. A step is ragged: sequence b brings q_start[b+1] - q_start[b] tokens after ctx[b] earlier ones and
+// owns state slot slots[b]; ctx 0 starts from zeros (m from 0) whatever the slot held, so slots change hands without clearing.
+// The running maximum is kept once per column block (mstate [slots, H, kScanMaxBlocks]), so that no workgroup reads what
+// another one writes.
+#include "common.h"
+#include "launch.h"
+
+namespace dlia {
+
+constexpr int kScanRows = 16;            // state rows per lane
+constexpr int kScanMaxBlocks = 128;      // copies of the running maximum per (slot, head)
+
+struct ScanArgs {
+  float* o; long ldo;
+  const float* z; long ldz;
+  const float* wz; long ldw;
+  float* state; float* mstate;
+  const float* b0; const float* b1;
+  const int* q_start; const int* ctx; const int* slots;
+  int H, d, dv, NC, R, CB, CH, DP, state_rows;
+  int col_q, col_k, col_v, col_a, col_i, col_f;
+  float cap, qscale;
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float logsigmoidf_(float x) { return x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x)); }
+
+template <int RULE>
+__global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
+  extern __shared__ float lds[];
+  constexpr int NV = RULE == 0 ? 5 : 2;
+  const int b = blockIdx.x, h = blockIdx.y, zb = blockIdx.z;
+  const int t0 = p.q_start[b], n = p.q_start[b + 1] - t0, c0 = p.ctx[b], slot = p.slots[b];
+  if (n <= 0 || slot < 0 || slot >= p.state_rows) return;
+  const int tid = threadIdx.x, R = p.R, CB = p.CB, DP = p.DP, d = p.d, NC = p.NC;
+  const int c = tid / R, rg = tid % R, j = zb * CB + c;
+  const bool col_ok = j < NC;
+  float* vec = lds;                                  // [CH][NV][DP]
+  float* vals = vec + (long)p.CH * NV * DP;          // [CH][CB]
+  float* sc = vals + (long)p.CH * CB;                // [CH][4]: rule 1: log i, log f -> keep, put, exp(-m')
+  float* S = p.state + ((long)slot * p.H + h) * (long)d * NC;
+  float s[kScanRows];
+#pragma unroll
+  for (int e = 0; e < kScanRows; ++e) {
+    const int row = rg * kScanRows + e;
+    s[e] = (c0 > 0 && col_ok && row < d) ? S[(long)row * NC + j] : 0.f;
+  }
+  float* mp = p.mstate ? p.mstate + ((long)slot * p.H + h) * kScanMaxBlocks + zb : nullptr;
+  float m_run = (RULE == 1 && c0 > 0) ? mp[0] : 0.f;         // (only thread 0's copy is used)
+  const int tt = tid >> 4, sub = tid & 15;
+  const int hd = h * d;
+  for (int ch0 = 0; ch0 < n; ch0 += p.CH) {
+    const int nt = min(p.CH, n - ch0);
+    __syncthreads();                                 // the previous chunk has been consumed
+    if (tt < nt) {
+      const long t = t0 + ch0 + tt;
+      const float* zr = p.z + t * p.ldz;
+      float* v0 = vec + (long)tt * NV * DP;
+      if constexpr (RULE == 0) {
+        const float* wr = p.wz + t * p.ldw;
+        float ksq = 0.f;
+        for (int i = sub; i < DP; i += 16) {
+          float k = 0.f, r = 0.f, a = 0.f, w = 0.f;
+          if (i < d) {
+            k = zr[p.col_k + hd + i]; r = zr[p.col_q + hd + i];
+            a = sigmoidf_(zr[p.col_a + hd + i] + p.b0[hd + i]);
+            w = expf(-0.6065306597126334f * sigmoidf_(wr[hd + i] + p.b1[hd + i]));
+          }
+          ksq += k * k;
+          v0[i] = w; v0[DP + i] = a; v0[3 * DP + i] = k; v0[4 * DP + i] = r;
+        }
+#pragma unroll
+        for (int o = 8; o >= 1; o >>= 1) ksq += __shfl_xor(ksq, o, 64);
+        const float inv = rsqrtf(ksq + 1e-6f);
+        for (int i = sub; i < DP; i += 16) {          // (each lane re-reads what it wrote itself)
+          const float u = v0[3 * DP + i] * inv;
+          v0[DP + i] *= u; v0[2 * DP + i] = u;
+        }
+      } else {
+        for (int i = sub; i < DP; i += 16) {
+          v0[i] = i < d ? zr[p.col_k + hd + i] : 0.f;
+          v0[DP + i] = i < d ? zr[p.col_q + hd + i] * p.qscale : 0.f;
+        }
+        if (sub == 0) {
+          sc[tt * 4] = p.cap * tanhf((zr[p.col_i + h] + p.b0[h]) / p.cap);
+          sc[tt * 4 + 1] = logsigmoidf_(p.cap * tanhf((zr[p.col_f + h] + p.b0[p.H + h]) / p.cap));
+        }
+      }
+      for (int cc = sub; cc < CB; cc += 16) {
+        const int jj = zb * CB + cc;
+        float v = 0.f;
+        if (jj < p.dv) v = zr[p.col_v + h * p.dv + jj];
+        else if (RULE == 1 && jj == p.dv) v = 1.f;
+        vals[tt * CB + cc] = v;
+      }
+    }
+    if constexpr (RULE == 1) {
+      __syncthreads();
+      if (tid == 0)
+        for (int q = 0; q < nt; ++q) {
+          const float li = sc[q * 4], lf = sc[q * 4 + 1];
+          const float m_new = fmaxf(lf + m_run, li);
+          sc[q * 4] = expf(lf + m_run - m_new); sc[q * 4 + 1] = expf(li - m_new); sc[q * 4 + 2] = expf(-m_new);
+          m_run = m_new;
+        }
+    }
+    __syncthreads();
+    for (int q = 0; q < nt; ++q) {
+      const float* v0 = vec + (long)q * NV * DP + rg * kScanRows;
+      const float v = vals[q * CB + c];
+      float out = 0.f;
+      if constexpr (RULE == 0) {
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < kScanRows; ++e) dot += v0[2 * DP + e] * s[e];
+        for (int o = 1; o < R; o <<= 1) dot += __shfl_xor(dot, o, 64);
+#pragma unroll
+        for (int e = 0; e < kScanRows; ++e) {
+          s[e] = v0[e] * s[e] - v0[DP + e] * dot + v0[3 * DP + e] * v;
+          out += v0[4 * DP + e] * s[e];
+        }
+      } else {
+        const float keep = sc[q * 4], put = sc[q * 4 + 1] * v;
+#pragma unroll
+        for (int e = 0; e < kScanRows; ++e) {
+          s[e] = keep * s[e] + put * v0[e];
+          out += v0[DP + e] * s[e];
+        }
+      }
+      for (int o = 1; o < R; o <<= 1) out += __shfl_xor(out, o, 64);
+      if (rg == 0 && col_ok) {
+        float* orow = p.o + (long)(t0 + ch0 + q) * p.ldo;
+        if constexpr (RULE == 0) orow[h * p.dv + j] = out;
+        else {
+          orow[h * (p.dv + 2) + j] = out;
+          if (j == p.dv) orow[h * (p.dv + 2) + p.dv + 1] = sc[q * 4 + 2];
+        }
+      }
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int e = 0; e < kScanRows; ++e) {
+      const int row = rg * kScanRows + e;
+      if (row < d) S[(long)row * NC + j] = s[e];
+    }
+  }
+  if (RULE == 1 && tid == 0) mp[0] = m_run;
+}
+
+}  // namespace dlia
+
+// Column blocks a (d, columns) state is split into: the launch shape depends on the sizes only, never on the step.
+extern "C" int dlia_state_scan_blocks(int d, int ncols) {
+  int R = 1;
+  while (R * dlia::kScanRows < d) R <<= 1;
+  if (R > 64) return -1;
+  const int CB = 256 / R;
+  return (ncols + CB - 1) / CB;
+}
+
+extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, const float* wz, long ldw, float* state,
+                               float* mstate, const float* b0, const float* b1, const int* q_start, const int* ctx,
+                               const int* slots, int B, int H, int d, int dv, int state_rows, int col_q, int col_k, int col_v,
+                               int col_a, int col_i, int col_f, float cap, float qscale, hipStream_t stream) {
+  if (B <= 0) return 0;
+  dlia::ScanArgs p;
+  p.o = o; p.ldo = ldo; p.z = z; p.ldz = ldz; p.wz = wz; p.ldw = ldw; p.state = state; p.mstate = mstate; p.b0 = b0; p.b1 = b1;
+  p.q_start = q_start; p.ctx = ctx; p.slots = slots; p.H = H; p.d = d; p.dv = dv; p.NC = rule == 0 ? dv : dv + 1;
+  int R = 1;
+  while (R * dlia::kScanRows < d) R <<= 1;
+  if (R > 64) return 1;
+  p.R = R; p.CB = 256 / R; p.DP = R * dlia::kScanRows; p.state_rows = state_rows;
+  const int nv = rule == 0 ? 5 : 2;
+  const int per_token = nv * p.DP + p.CB + 4;
+  int CH = 12000 / per_token;
+  p.CH = CH > 16 ? 16 : (CH < 1 ? 1 : CH);
+  p.col_q = col_q; p.col_k = col_k; p.col_v = col_v; p.col_a = col_a; p.col_i = col_i; p.col_f = col_f; p.cap = cap; p.qscale = qscale;
+  const int ZB = (p.NC + p.CB - 1) / p.CB;
+  if (ZB > dlia::kScanMaxBlocks) return 2;
+  const size_t lds = (size_t)p.CH * per_token * sizeof(float);
+  const dim3 grid(B, H, ZB);
+  if (rule == 0)
+    hipLaunchKernelGGL(dlia::state_scan_kernel<0>, grid, dim3(256), lds, stream, p);
+  else
+    hipLaunchKernelGGL(dlia::state_scan_kernel<1>, grid, dim3(256), lds, stream, p);
+  return 0;
+}

@@ -1,7 +1,8 @@
 // Paged attention for mixers whose sizes and mask are free parameters: queries / keys of `d`, values of `dv`
 // (any sizes), an optional sliding window (a query at position i sees the keys j with 0 <= i - j < window), an
-// optional softmax sink (one more term exp(0) in the denominator, with no value), no rotation, the score scale
-// given. Scores, the softmax and the weighted sum are fp32; the cache holds the compute type (bf16 or fp32).
+// optional softmax sink (one more term exp(0), or exp of a learned number per head, in the denominator, with no value),
+// no rotation, the score scale given. Optional per head: a learned factor on the scaled scores, a bias per distance i - j
+// (a table [distances, heads], added after scale and factor), a sigmoid gate on the head's output (one logit per token, head). Scores, the softmax and the weighted sum are fp32; the cache holds the compute type (bf16 or fp32).
 //
 // Cache layout per layer: K [block][kv head][32][d], V [block][kv head][32][dv], plain rows, blocks of 32 tokens
 // addressed through the stage's block table (the same table and block ids as every other layer's cache).
@@ -57,7 +58,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     OT* __restrict__ out, const float* __restrict__ qkv, const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, const int* __restrict__ block_table, int items,
     int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv, long ldq, long ldo, float scale, int window,
-    int sink) {
+    int sink, const float* __restrict__ temp, const float* __restrict__ bias, int bias_rows, const float* __restrict__ sinkv,
+    const float* __restrict__ gate, long ldg) {
   __shared__ float qs[4][kWinMaxD];
   const int wave = threadIdx.x >> 6, lane = lane_id();
   const int item = blockIdx.x * 4 + wave;
@@ -71,11 +73,12 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     return;
   }
   const float* qrow = qkv + (long)t * ldq + (long)h * d;
-  for (int i = lane; i < d; i += 64) qs[wave][i] = qrow[i] * scale;
+  const float hscale = temp ? scale * temp[h] : scale;
+  for (int i = lane; i < d; i += 64) qs[wave][i] = qrow[i] * hscale;
   __builtin_amdgcn_wave_barrier();
   const int* table = block_table + (long)slot * max_blocks;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float m = sink ? (sinkv ? sinkv[h] : 0.f) : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[kWinMaxD / 64];
 #pragma unroll
   for (int c = 0; c < kWinMaxD / 64; ++c) acc[c] = 0.f;
@@ -90,6 +93,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       const T* krow = kcache + (((long)blk * G + g) * kWinBlock + (j % kWinBlock)) * d;
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot += qs[wave][i] * (float)krow[i];
+      if (bias) dot += bias[(long)min(pos - j, bias_rows - 1) * H + h];
       s = dot;
     }
     const float cm = wave_max(s);
@@ -112,7 +116,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
         if (c < ncol) { const int col = c * 64 + lane; if (col < dv) acc[c] += pj * (float)vrow[col]; }
     }
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float inv = l > 0.f ? 1.f / l : 0.f;
+  if (gate) inv *= 1.f / (1.f + expf(-gate[(long)t * ldg + h]));
 #pragma unroll
   for (int c = 0; c < kWinMaxD / 64; ++c)
     if (c < ncol) { const int col = c * 64 + lane; if (col < dv) orow[col] = (OT)(acc[c] * inv); }
@@ -158,16 +163,17 @@ extern "C" void dlia_kv_store(const float* qkv, float* vfirst, const float* lam,
 extern "C" void dlia_window_attention(void* out, const float* qkv, const void* kcache, const void* vcache, int f32,
                                       const int* tok_pos, const int* tok_seq, const int* block_table, int T, int max_blocks,
                                       int num_blocks, int table_rows, int H, int G, int d, int dv, long ldq, long ldo,
-                                      float scale, int window, int sink, hipStream_t stream) {
+                                      float scale, int window, int sink, const float* temp, const float* bias, int bias_rows,
+                                      const float* sinkv, const float* gate, long ldg, hipStream_t stream) {
   const int items = T * H;
   if (items <= 0) return;
   const dim3 grid((items + 3) / 4);
   if (f32)
     hipLaunchKernelGGL((dlia::window_attention_kernel<float, float>), grid, dim3(256), 0, stream, (float*)out, qkv,
                        (const float*)kcache, (const float*)vcache, tok_pos, tok_seq, block_table, items, max_blocks, num_blocks,
-                       table_rows, H, G, d, dv, ldq, ldo, scale, window, sink);
+                       table_rows, H, G, d, dv, ldq, ldo, scale, window, sink, temp, bias, bias_rows, sinkv, gate, ldg);
   else
     hipLaunchKernelGGL((dlia::window_attention_kernel<dlia::bf16, dlia::bf16>), grid, dim3(256), 0, stream, (dlia::bf16*)out, qkv,
                        (const dlia::bf16*)kcache, (const dlia::bf16*)vcache, tok_pos, tok_seq, block_table, items, max_blocks,
-                       num_blocks, table_rows, H, G, d, dv, ldq, ldo, scale, window, sink);
+                       num_blocks, table_rows, H, G, d, dv, ldq, ldo, scale, window, sink, temp, bias, bias_rows, sinkv, gate, ldg);
 }
