@@ -1,4 +1,5 @@
-"""Prefill and decode throughput of a Letarax stack beside a Llama stack of equal size (`bench.py --hybrid-compare`).
+"""Prefill and decode throughput of a Letarax stack beside a Llama stack of equal size (`bench.py --hybrid-compare`), and of a
+Nufapel stack beside the Letarax stack of equal size (`bench.py --gated-compare`).
 
 Both models get random weights and the same width, head counts, head size, feed-forward width, depth and
 vocabulary; the Letarax stack has three attention layers (windowed, with the sink and value mixing) to one delta-rule
@@ -18,6 +19,13 @@ SIZES = {
     "8b-like": (4096, 32, 8, 128, 14336, 4, 2048),
 }
 VOCAB = 32000
+
+
+def gated_specs(name: str):
+    """The Nufapel stack of a size beside the closest existing design of the same size: the Letarax stack (both keep an fp32
+    residual stream, attention over the paged cache beside recurrent layers with slot-resident state)."""
+    from distributed_llm_inference_amd.models.spec import BUILTIN_SPECS
+    return BUILTIN_SPECS[f"nufapel-{name}"], BUILTIN_SPECS[f"letarax-{name}"]
 
 
 def specs(name: str):
@@ -84,21 +92,21 @@ def time_decode(ex, rows: int, ctx: int, iters: int) -> float:
     return e0.elapsed_time(e1) / 1e3 / iters
 
 
-def main(sizes=None, iters: int = 8, out=sys.stdout) -> int:
+def main(sizes=None, iters: int = 8, out=sys.stdout, gated: bool = False) -> int:
     import gc
     import torch
     rows, ctx, plen = 64, 1024, 2048
     for name in (sizes or list(SIZES)):
-        rec = {"metric": "letarax_vs_llama_tokens_per_s", "size": name, "dtype": "bf16", "data": "synthetic", "weights": "random",
+        rec = {"metric": "nufapel_vs_letarax_tokens_per_s" if gated else "letarax_vs_llama_tokens_per_s", "size": name, "dtype": "bf16", "data": "synthetic", "weights": "random",
                "config": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "layers", "window"), SIZES[name])),
                "prefill": {"prompts": 1, "tokens": plen}, "decode": {"rows": rows, "context": ctx}}
-        for spec in specs(name):
+        for spec in (gated_specs(name) if gated else specs(name)):
             t0 = time.perf_counter()
             ex = build(spec, rows, plen, max(plen, ctx + 256))
             tp = time_prefill(ex, 1, plen, iters)
             td = time_decode(ex, rows, ctx, 4 * iters)
             tl = time_decode(ex, rows, 64, 4 * iters)
-            key = "letarax" if spec.is_hybrid else "llama"
+            key = spec.family
             rec[key] = {"prefill_tok_s": round(plen / tp, 1), "prefill_ms": round(tp * 1e3, 3),
                         "decode_tok_s": round(rows / td, 1), "decode_ms": round(td * 1e3, 3),
                         "decode_short_ctx_ms": round(tl * 1e3, 3), "bringup_s": round(time.perf_counter() - t0, 1)}
@@ -106,8 +114,9 @@ def main(sizes=None, iters: int = 8, out=sys.stdout) -> int:
             del ex
             gc.collect()
             torch.cuda.empty_cache()
-        rec["prefill_ratio"] = round(rec["letarax"]["prefill_tok_s"] / rec["llama"]["prefill_tok_s"], 3)
-        rec["decode_ratio"] = round(rec["letarax"]["decode_tok_s"] / rec["llama"]["decode_tok_s"], 3)
+        new, old = ("nufapel", "letarax") if gated else ("letarax", "llama")
+        rec["prefill_ratio"] = round(rec[new]["prefill_tok_s"] / rec[old]["prefill_tok_s"], 3)
+        rec["decode_ratio"] = round(rec[new]["decode_tok_s"] / rec[old]["decode_tok_s"], 3)
         out.write(json.dumps(rec) + "\n")
         out.flush()
     return 0

@@ -107,6 +107,15 @@ class LayerSpec:
     def has_ff(self) -> bool:
         return self.ff > 0 or self.moe is not None
 
+    @property
+    def qk_heads(self) -> int:
+        """Heads of the q projection: every query head for attention, the shared q / k heads for the delta rule."""
+        return self.heads if self.kind == "attention" else self.kv_heads
+
+    @property
+    def v_heads(self) -> int:
+        return self.kv_heads if self.kind == "attention" else self.heads
+
     def mixer_param_count(self, width: int) -> int:
         if self.kind == "parallel":
             return sum(b.mixer_param_count(width) + width for b in self.branches)
@@ -686,9 +695,32 @@ def letarax_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
                      tie_embeddings=True, bos_token_id=1, eos_token_id=2, hf_type="letarax", layer_specs=layers)
 
 
+def nufapel_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int, ff: int, num_layers: int, vocab_size: int = 32000,
+                 pattern: str = "pgpp", experts: int = 8, top: int = 2, loop: tuple = (), max_position: int = 8192, rank: int = 64,
+                 bias_rows: int = 32, bias_max: int = 2048) -> ModelSpec:
+    """A Nufapel stack from a few numbers: `pattern` repeats over the layers ('p': attention with distance bias, head temperature,
+    learned sink and head gate beside a matrix memory of half as many heads; 'g': generalised delta rule over width / head_dim
+    heads); 'g' layers have a dense feed-forward of `ff`, 'p' layers a routed one of `experts` experts of ff / 4, `top` chosen."""
+    moe = MoeSpec(experts=experts, top=top, ff=max(8, ff // 4), groups=max(1, experts // 4), keep=max(1, experts // 8), scale=1.0, limit=7.0)
+    left = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5, sink=True,
+                     sink_learned=True, head_temp=True, head_gate=True, bias_rows=bias_rows, bias_max=bias_max)
+    right = LayerSpec("mlstm", heads=max(1, heads // 2), kv_heads=max(1, heads // 2), dim=head_dim, vdim=head_dim, gate_cap=15.0, scale=head_dim ** -0.5)
+    par = LayerSpec("parallel", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, branches=(left, right), ff=0, ff_kind="moe", moe=moe)
+    gh = max(1, width // head_dim)
+    gd = LayerSpec("general_delta", heads=gh, kv_heads=gh, dim=head_dim, vdim=head_dim, rank=rank, ff=ff, ff_kind="gelu")
+    layers = tuple(par if pattern[i % len(pattern)] == "p" else gd for i in range(num_layers))
+    return ModelSpec(name=name, family="nufapel", num_layers=num_layers, hidden_size=width, num_heads=heads, num_kv_heads=kv_heads,
+                     head_dim=head_dim, intermediate_size=ff, vocab_size=vocab_size, max_position=max_position, norm_eps=1e-5,
+                     tie_embeddings=False, bos_token_id=1, eos_token_id=2, hf_type="nufapel", layer_specs=layers, norm_kind="dyt",
+                     gated_residual=True, loop=loop, learned_positions=True, logit_softcap=30.0)
+
+
 # Letarax stacks of the sizes of the Llama benchmark shapes (random weights; `bench.py --hybrid-compare` runs them)
 BUILTIN_SPECS["letarax-1b-like"] = letarax_spec("letarax-1b-like", 2048, 16, 4, 128, 8192, 8, 1024)
 BUILTIN_SPECS["letarax-8b-like"] = letarax_spec("letarax-8b-like", 4096, 32, 8, 128, 14336, 4, 2048)
+# Nufapel stacks of the same sizes (`bench.py --gated-compare` runs them beside the Letarax stacks)
+BUILTIN_SPECS["nufapel-1b-like"] = nufapel_spec("nufapel-1b-like", 2048, 16, 4, 128, 8192, 8)
+BUILTIN_SPECS["nufapel-8b-like"] = nufapel_spec("nufapel-8b-like", 4096, 32, 8, 128, 14336, 4)
 
 
 def _register_test_models():
@@ -704,6 +736,10 @@ def _register_test_models():
         intermediate_size=512, vocab_size=320, num_layers=4, hf_type="qwen2", qkv_bias=True, tie_embeddings=True)
     BUILTIN_SPECS["tiny-letarax-test"] = letarax_spec("tiny-letarax-test", 64, 4, 2, 16, 96, 4, 12, vocab_size=320, conv=3, pattern="ada")
     BUILTIN_SPECS["tiny-letarax-gpu-test"] = letarax_spec("tiny-letarax-gpu-test", 128, 4, 2, 64, 256, 4, 40, vocab_size=320)
+    BUILTIN_SPECS["tiny-nufapel-test"] = nufapel_spec("tiny-nufapel-test", 64, 4, 2, 16, 96, 3, vocab_size=320, pattern="pgp", experts=4,
+                                                      loop=(0, 2, 2), max_position=256, rank=8, bias_rows=8, bias_max=64)
+    BUILTIN_SPECS["tiny-nufapel-gpu-test"] = nufapel_spec("tiny-nufapel-gpu-test", 128, 4, 2, 32, 256, 4, vocab_size=320, experts=8,
+                                                          loop=(1, 3, 2), max_position=512, rank=16, bias_rows=16, bias_max=200)
     BUILTIN_SPECS["tiny-gpt2-gpu-test"] = tiny_spec(
         "gpt2", name="tiny-gpt2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=4, head_dim=64,
         intermediate_size=1024, vocab_size=333, num_layers=4)

@@ -114,10 +114,9 @@ class HybridGpuStage(GpuStage):
                           for ls in self.specs]
         self._no_rope = {D: torch.zeros(1, D // 2, device=self.device) for D in (64, 128)}
         if spec.norm_kind == "dyt":
-            # one cache / state per layer RUN; the attention of these stacks (distance bias, temperatures, learned sinks, head
-            # gates) runs on the any-size kernel
+            # one cache / state per layer RUN
             self._attn_of_run = [spec.layer_specs[li].branches[0] if spec.layer_specs[li].kind == "parallel" else None for li, _ in spec.layer_runs()]
-            self.mfma_attn = [False] * len(self._attn_of_run)
+            self.mfma_attn = [mfma_ok and a is not None and a.dim == a.vdim and a.dim in (64, 128) and a.group <= 16 for a in self._attn_of_run]
         else:
             self._attn_of_run = [ls if ls.kind == "attention" else None for ls in self.specs]
         self.gated = spec.norm_kind == "dyt"
@@ -316,7 +315,7 @@ class HybridGpuStage(GpuStage):
     def _layers(self, wk: _HybridWork, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int, splits: int,
                 alone: bool = False, lead_decode: int = 0):
         if self.gated:
-            return self._layers_gated(wk, T, tok_pos, tok_seq, q_start, ctx, slots)
+            return self._layers_gated(wk, T, B, tok_pos, tok_seq, q_start, ctx, slots, max_q, lead_decode)
         K, eps = self.K, self.spec.norm_eps
         h, xn, yo = wk.h[:T], wk.xn[:T], wk.yo[:T]
         view = lambda buf, cols: buf[:T * cols].view(T, cols)
@@ -408,7 +407,17 @@ class HybridGpuStage(GpuStage):
             l = weights.layers[i]
             p = {k: f32(l[k]) for k in ("ln1_w", "ln1_b", "b_rg1", "o_norm_w")}
             p["ln1_a"] = float(l["ln1_a"])
-            self._matrix(p, "w_in", torch.cat([mat(l["w_in"]), mat(l["w_rg1"])]), None)
+            w_in = mat(l["w_in"])
+            p["fast"] = False
+            if ls.kind == "parallel":
+                a = ls.branches[0]
+                run = [ri for ri, (li, _) in enumerate(self.runs) if li == i][0]
+                if self.mfma_attn[run]:
+                    # q | k | v of the attention leave through a GEMM of their own, in bf16, for the MFMA attention kernels
+                    c = (a.heads + a.kv_heads) * a.dim + a.kv_heads * a.vdim
+                    self._matrix(p, "w_qkv", w_in[:c].contiguous(), None)
+                    w_in, p["fast"] = w_in[c:], True
+            self._matrix(p, "w_in", torch.cat([w_in, mat(l["w_rg1"])]), None)
             self._matrix(p, "w_o", mat(l["w_o"]), None)
             if ls.kind == "general_delta":
                 p["rank"] = int(l["w_w2"].shape[1])
@@ -419,6 +428,8 @@ class HybridGpuStage(GpuStage):
                 p["bias"] = R.distance_bias_table(l["rel"].float().cpu(), a.bias_max, self.max_seq_len).to(dev).contiguous()
                 for k in ("temp", "sink", "b_if", "out_l", "out_r"):
                     p[k] = f32(l[k])
+                if p["fast"]:                        # (the MFMA kernels keep scores in the units of q . k)
+                    p["bias"], p["sink"] = (p["bias"] / a.scale).contiguous(), (p["sink"] / a.scale).contiguous()
                 self._matrix(p, "w_o_r", mat(l["w_o_r"]), None)
             if ls.has_ff:
                 p.update({k: f32(l[k]) for k in ("ln2_w", "ln2_b", "b_rg2")})
@@ -441,10 +452,12 @@ class HybridGpuStage(GpuStage):
         s, dev, at = self.spec, self.device, self.act_dtype
         z = lambda n, dt=torch.float32: torch.zeros(max(int(n), 1), device=dev, dtype=dt)
         B, H = min(rows, self.max_batch), s.hidden_size
-        zc = wc = lc = oc = mc = m2 = z2 = ac = yc = 1
+        zc = wc = lc = oc = mc = m2 = z2 = ac = yc = qc = 1
         pairs = tiles = ef = 0
         for ls, p in zip(self.specs, self.layers):
             zc, yc = max(zc, self._cols(p, "w_in")), max(yc, self._cols(p, "w_o"))
+            if p["fast"]:
+                qc = max(qc, self._cols(p, "w_qkv"))
             if ls.kind == "general_delta":
                 n = ls.heads * ls.dim
                 wc, lc, oc, mc = max(wc, self._cols(p, "w_w2")), max(lc, p["rank"]), max(oc, n), max(mc, n)
@@ -470,9 +483,10 @@ class HybridGpuStage(GpuStage):
             low=z(rows * lc, at), o=z(rows * oc), mixed=z(rows * mc, at), mixed2=z(rows * m2, at), ya=z(rows * yc), yb=z(rows * yc),
             z2=z(rows * z2), act=z(rows * ac, at), sel=z(pairs, i32), wts=z(pairs), pair_row=z(pairs, i32), tiles=z(1 + tiles, i32),
             row_tok=z(16 * tiles, i32), eact=z(16 * tiles * ef, at), ey=z(16 * tiles * H), ws=z(ws_floats + 4096),
+            qkv16=z(rows * qc, torch.bfloat16),
             head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
 
-    def _layers_gated(self, wk, T: int, tok_pos, tok_seq, q_start, ctx, slots):
+    def _layers_gated(self, wk, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int, lead_decode: int):
         K, eps, H = self.K, self.spec.norm_eps, self.spec.hidden_size
         h, xn = wk.h[:T], wk.xn[:T]
         view = lambda buf, cols: buf[:T * cols].view(T, cols)
@@ -509,14 +523,30 @@ class HybridGpuStage(GpuStage):
             else:
                 a, b = ls.branches
                 qn, kn, vn, bn, bv = a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, b.heads * b.dim, b.heads * b.vdim
-                c_g = qn + kn + vn
+                c_g = 0 if p["fast"] else qn + kn + vn       # (z starts behind q | k | v when they have a GEMM of their own)
                 c_q = c_g + a.heads
                 c_k, c_v, c_rg, c_i = c_q + bn, c_q + 2 * bn, c_q + 2 * bn + bv, c_q + 2 * bn + 2 * bv
-                kc, vc = self.kv[ri]
                 mixed, mixed2, o = view(wk.mixed, a.heads * a.vdim), view(wk.mixed2, bv), view(wk.o, b.heads * (b.vdim + 2))
-                K.kv_store(z[:, :c_g], None, None, 0, kc, vc, tok_pos, tok_seq, self.block_table, a.kv_heads, a.dim, a.vdim, qn)
-                K.biased_attention(mixed, z, kc, vc, tok_pos, tok_seq, self.block_table, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
-                                   p["temp"], p["bias"], p["sink"], z[:, c_g:c_q])
+                gate = z[:, c_g:c_q]
+                if p["fast"]:
+                    Ha, G, d = a.heads, a.kv_heads, a.dim
+                    qkv = view(wk.qkv16, self._cols(p, "w_qkv"))
+                    self._mm(wk, qkv, xn, p, "w_qkv")
+                    K.rope_kvwrite(qkv, None, 1, None, self.kv[ri], self._no_rope[d], self._no_rope[d], tok_pos, tok_seq,
+                                   self.block_table, Ha, G, d, False)
+                    ext = (p["temp"], p["bias"], p["sink"], gate)
+                    if 0 < lead_decode < B and max_q > 1:
+                        # single tokens riding in front of prompt portions: the decode-shaped kernel for them, the prefill-shaped for the rest
+                        n = lead_decode
+                        K.paged_attention_biased(mixed, qkv, self.kv[ri], q_start[:n + 1], ctx[:n], self.block_table, slots[:n], 1, Ha, G, d, a.scale, *ext)
+                        K.paged_attention_biased(mixed, qkv, self.kv[ri], q_start[n:], ctx[n:], self.block_table, slots[n:], max_q, Ha, G, d, a.scale, *ext)
+                    else:
+                        K.paged_attention_biased(mixed, qkv, self.kv[ri], q_start, ctx, self.block_table, slots, max_q, Ha, G, d, a.scale, *ext)
+                else:
+                    kc, vc = self.kv[ri]
+                    K.kv_store(z[:, :c_g], None, None, 0, kc, vc, tok_pos, tok_seq, self.block_table, a.kv_heads, a.dim, a.vdim, qn)
+                    K.biased_attention(mixed, z, kc, vc, tok_pos, tok_seq, self.block_table, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
+                                       p["temp"], p["bias"], p["sink"], gate)
                 self._mm(wk, ya, mixed, p, "w_o")
                 K.state_scan(1, o, z, None, self.rec[ri][0], self.rec[ri][1], p["b_if"], None, q_start, ctx, slots, b.heads, b.dim, b.vdim,
                              c_q, c_k, c_v, 0, c_i, c_i + b.heads, b.gate_cap, b.scale)

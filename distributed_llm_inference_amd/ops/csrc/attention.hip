@@ -58,6 +58,12 @@ struct AttnParams {
   // context); sink: the softmax's denominator has one more term exp(0) that carries no value (added once, where
   // the row is normalised, so split and merged partials stay plain).
   int window, sink;
+  // Learned extras of the windowed / sink instantiations (all optional, per query head): `temp` multiplies a head's scores,
+  // `bias` [bias_rows, Hq] is added per distance i - j (distances beyond the table take its last row), `sinkv` is the sink's
+  // score instead of 0; bias and sinkv come divided by the softmax scale, so that every score stays in the units of q . k.
+  // `gate` [T, ldg]: the head's output is multiplied by sigmoid(gate[row, head]).
+  const float* temp; const float* bias; const float* sinkv; const float* gate;
+  int bias_rows; long ldg;
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -103,6 +109,17 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
     col_qpos[nt] = (tile_live && qp < q_len && hl < p.g_real) ? qp : -1;
     col_row[nt] = (long)(t0 + (qp < q_len ? qp : 0));
     col_head[nt] = kvh * p.g_real + hl;
+  }
+  [[maybe_unused]] float col_temp[NT], col_sink[NT];
+  [[maybe_unused]] const float* col_bias[NT];
+  if constexpr (WIN) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int hc = min(col_head[nt], p.Hq - 1);           // (padding columns stay inside the tables)
+      col_temp[nt] = p.temp ? p.temp[hc] : 1.f;
+      col_sink[nt] = p.sinkv ? p.sinkv[hc] : 0.f;
+      col_bias[nt] = p.bias ? p.bias + hc : nullptr;
+    }
   }
 
   // kv block range of this split; the 4 waves of the workgroup interleave its blocks.
@@ -207,6 +224,17 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
     for (int nt = 0; nt < NT; ++nt) {
       const int limit = col_qpos[nt] >= 0 ? ctx + col_qpos[nt] : -1;   // last visible key position
       float mx = kNegInf;
+      if constexpr (WIN) {
+        if (p.temp || p.bias) {
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int dist = min(max(limit - (kb * kBlockTokens + kt * 16 + quad * 4 + r), 0), p.bias_rows - 1);
+              st[kt][nt][r] = st[kt][nt][r] * col_temp[nt] + (col_bias[nt] ? col_bias[nt][(long)dist * p.Hq] : 0.f);
+            }
+        }
+      }
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -284,9 +312,12 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
       lt += __shfl_xor(lt, 32, 64);
       if (col_qpos[nt] < 0) continue;
       if constexpr (WIN) {
-        if (p.sink && p.splits == 1) lt += exp2f((0.f - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
+        if (p.sink && p.splits == 1) lt += exp2f((col_sink[nt] - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
       }
-      const float inv = lt > 0.f ? 1.f / lt : 0.f;
+      float inv = lt > 0.f ? 1.f / lt : 0.f;
+      if constexpr (WIN) {
+        if (p.gate) inv *= 1.f / (1.f + expf(-p.gate[col_row[nt] * p.ldg + col_head[nt]]));
+      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         const f32x4 acc = o[dt][nt];
@@ -337,9 +368,12 @@ __device__ __forceinline__ void paged_attn_body(const AttnParams& p, long item) 
     }
     if (col_qpos[nt] < 0) continue;
     if constexpr (WIN) {
-      if (p.sink && p.splits == 1) lt += exp2f((0.f - m_safe) * p.scale_log2);
+      if (p.sink && p.splits == 1) lt += exp2f((col_sink[nt] - m_safe) * p.scale_log2);
     }
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    float inv = lt > 0.f ? 1.f / lt : 0.f;
+    if constexpr (WIN) {
+      if (p.gate) inv *= 1.f / (1.f + expf(-p.gate[col_row[nt] * p.ldg + col_head[nt]]));
+    }
     for (int dt = wave; dt < DT; dt += 4) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -516,6 +550,16 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
     const int qp = qp0 + ((wave * 32 + nt * 16 + l15) >> p.g_shift);
     col_qpos[nt] = (tile_live && qp < q_len && ((wave * 32 + nt * 16 + l15) & (g - 1)) < p.g_real) ? qp : -1;
   }
+  [[maybe_unused]] float col_temp[NT];
+  [[maybe_unused]] const float* col_bias[NT];
+  if constexpr (WIN) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int hc = min(kvh * p.g_real + ((wave * 32 + nt * 16 + l15) & (g - 1)), p.Hq - 1);
+      col_temp[nt] = p.temp ? p.temp[hc] : 1.f;
+      col_bias[nt] = p.bias ? p.bias + hc : nullptr;
+    }
+  }
   // wave-uniform: first and last query position of this wave's columns
   const int wq_first = qp0 + ((wave * 32) >> p.g_shift);
   const int wq_last = min(q_len - 1, qp0 + ((wave * 32 + 31) >> p.g_shift));
@@ -605,6 +649,18 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       float mx = kNegInf;
+      if constexpr (WIN) {
+        if (p.temp || p.bias) {
+          const int qabs = ctx + col_qpos[nt];
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int dist = min(max(qabs - (kb * kBlockTokens + kt * 16 + quad * 4 + r), 0), p.bias_rows - 1);
+              st[kt][nt][r] = st[kt][nt][r] * col_temp[nt] + (col_bias[nt] ? col_bias[nt][(long)dist * p.Hq] : 0.f);
+            }
+        }
+      }
       if constexpr (MASK) {
         const int limit = col_qpos[nt] >= 0 ? ctx + col_qpos[nt] : -1;   // last visible key position
 #pragma unroll
@@ -703,13 +759,17 @@ __global__ __launch_bounds__(256, 2) void prefill_attn_kernel(AttnParams p) {
   for (int nt = 0; nt < NT; ++nt) {
     float lt = quad_sum(l[nt]);
     if (col_qpos[nt] < 0) continue;
-    if constexpr (WIN) {
-      if (p.sink) lt += exp2f((0.f - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
-    }
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
     int le = lane;
     asm volatile("" : "+v"(le));                   // recompute from the lane id instead of keeping the prologue's values live
     const int ce = wave * 32 + nt * 16 + (le & 15);
+    [[maybe_unused]] const int he = kvh * p.g_real + (ce & (g - 1));
+    if constexpr (WIN) {
+      if (p.sink) lt += exp2f(((p.sinkv ? p.sinkv[min(he, p.Hq - 1)] : 0.f) - (m[nt] == kNegInf ? 0.f : m[nt])) * p.scale_log2);
+    }
+    float inv = lt > 0.f ? 1.f / lt : 0.f;
+    if constexpr (WIN) {
+      if (p.gate) inv *= 1.f / (1.f + expf(-p.gate[(long)(t0 + col_qpos[nt]) * p.ldg + he]));
+    }
     bf16* orow = p.out + (long)(t0 + col_qpos[nt]) * p.ldo + (kvh * p.g_real + (ce & (g - 1))) * D + (le >> 4) * 4;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -801,10 +861,13 @@ extern "C" void dlia_paged_attention(void* out, const void* qkv, const void* kv_
                                      const int* q_start, const int* ctx_lens, const int* block_table,
                                      const int* slots, float* partial, int B, int max_q_len, int Hq,
                                      int Hkv, int D, int table_rows, int max_blocks, int num_blocks,
-                                     long ldq, long ldo, float scale, int splits, hipStream_t stream, int window, int sink) {
+                                     long ldq, long ldo, float scale, int splits, hipStream_t stream, int window, int sink,
+                                     const float* temp, const float* bias, int bias_rows, const float* sinkv, const float* gate,
+                                     long ldg) {
   if (B <= 0 || max_q_len <= 0) return;
   AttnParams p;
   p.window = kv_scale ? 0 : window; p.sink = kv_scale ? 0 : sink;
+  p.temp = temp; p.bias = bias; p.bias_rows = bias ? bias_rows : 1; p.sinkv = sinkv; p.gate = gate; p.ldg = ldg;
   p.out = (bf16*)out; p.ldo = ldo; p.q = (const bf16*)qkv; p.ldq = ldq; p.kv = (const bf16*)kv_cache; p.kv_scale = kv_scale;
   p.q_start = q_start; p.ctx_lens = ctx_lens; p.block_table = block_table; p.slots = slots; p.table_rows = table_rows; p.partial = partial;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv;

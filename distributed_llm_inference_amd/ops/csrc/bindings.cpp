@@ -444,7 +444,9 @@ int64_t attention_ws_floats(int64_t B, int64_t max_q_len, int64_t Hq, int64_t Hk
 static void paged_attention_impl(Tensor out, const Tensor& qkv, const Tensor& kv_cache, OptTensor kv_scale,
                                  const Tensor& q_start, const Tensor& ctx_lens, const Tensor& block_table,
                                  OptTensor slots, OptTensor partial, int64_t max_q_len, int64_t Hq, int64_t Hkv,
-                                 int64_t D, double scale, int64_t splits, int64_t window = 0, bool sink = false) {
+                                 int64_t D, double scale, int64_t splits, int64_t window = 0, bool sink = false,
+                                 OptTensor temp = c10::nullopt, OptTensor bias = c10::nullopt, OptTensor sinkv = c10::nullopt,
+                                 OptTensor gate = c10::nullopt) {
   DLIA_ON_DEVICE_OF(out);
   check_bf16(out, "out"); check_bf16(qkv, "qkv"); check_rows(out, "out"); check_rows(qkv, "qkv");
   DLIA_CHECK(window >= 0 && (!kv_scale.has_value() || (window == 0 && !sink)), "window / sink: bf16 cache only, window >= 0");
@@ -476,13 +478,31 @@ static void paged_attention_impl(Tensor out, const Tensor& qkv, const Tensor& kv
   } else {
     sp = 1;
   }
+  const float *tp = nullptr, *bp = nullptr, *sk = nullptr, *gp = nullptr;
+  int brows = 0; long ldg = 0;
+  if (temp.has_value() || bias.has_value() || sinkv.has_value() || gate.has_value()) {
+    DLIA_CHECK(sink && sp == 1 && !kv_scale.has_value(), "learned attention extras: sink instantiation, no split, bf16 cache");
+    if (temp.has_value()) { check_f32(*temp, "temp"); DLIA_CHECK(temp->numel() == Hq, "temp [Hq]"); tp = temp->data_ptr<float>(); }
+    if (sinkv.has_value()) { check_f32(*sinkv, "sinkv"); DLIA_CHECK(sinkv->numel() == Hq, "sinkv [Hq]"); sk = sinkv->data_ptr<float>(); }
+    if (bias.has_value()) {
+      check_f32(*bias, "bias");
+      DLIA_CHECK(bias->dim() == 2 && bias->size(1) == Hq && bias->size(0) >= 1, "bias [distances, Hq]");
+      bp = bias->data_ptr<float>(); brows = (int)bias->size(0);
+    }
+    if (gate.has_value()) {
+      check_dev(*gate, "gate");
+      DLIA_CHECK(gate->scalar_type() == at::kFloat && gate->dim() == 2 && gate->stride(1) == 1 && gate->size(1) == Hq &&
+                 gate->size(0) >= out.size(0), "gate logits: float32 [T, Hq]");
+      gp = gate->data_ptr<float>(); ldg = gate->stride(0);
+    }
+  }
   // The caller guarantees: q_start is non-decreasing with q_start[B] <= rows of qkv/out, chunk
   // lengths <= max_q_len, and ctx_lens[b] + q_len[b] <= 32 * block_table.size(1).
   dlia_paged_attention(out.data_ptr(), qkv.data_ptr(), kv_cache.data_ptr(),
                        kv_scale.has_value() ? kv_scale->data_ptr<float>() : nullptr, q_start.data_ptr<int>(),
                        ctx_lens.data_ptr<int>(), block_table.data_ptr<int>(), slp, pp, (int)B, (int)max_q_len, (int)Hq,
                        (int)Hkv, (int)D, (int)block_table.size(0), (int)block_table.size(1), (int)geo.num_blocks, qkv.stride(0),
-                       out.stride(0), (float)scale, sp, cur_stream(), (int)window, sink ? 1 : 0);
+                       out.stride(0), (float)scale, sp, cur_stream(), (int)window, sink ? 1 : 0, tp, bp, brows, sk, gp, ldg);
 }
 
 // Causal attention restricted to a sliding window (0: none), optionally with a softmax sink, over the bf16 cache.
@@ -492,6 +512,15 @@ void paged_attention_window(Tensor out, const Tensor& qkv, const Tensor& kv_cach
                             int64_t window, bool sink) {
   paged_attention_impl(out, qkv, kv_cache, c10::nullopt, q_start, ctx_lens, block_table, slots, partial, max_q_len, Hq, Hkv, D,
                        scale, splits, window, sink);
+}
+
+// The sink instantiation with learned extras per query head: a factor on the scores, a bias per distance (both the bias and
+// the sink's score come divided by `scale`), the sink's score, a sigmoid gate on the output.
+void paged_attention_biased(Tensor out, const Tensor& qkv, const Tensor& kv_cache, const Tensor& q_start, const Tensor& ctx_lens,
+                            const Tensor& block_table, OptTensor slots, int64_t max_q_len, int64_t Hq, int64_t Hkv, int64_t D,
+                            double scale, OptTensor temp, OptTensor bias, OptTensor sinkv, OptTensor gate) {
+  paged_attention_impl(out, qkv, kv_cache, c10::nullopt, q_start, ctx_lens, block_table, slots, c10::nullopt, max_q_len, Hq, Hkv, D,
+                       scale, 1, 0, true, temp, bias, sinkv, gate);
 }
 
 void value_mix(Tensor qkv, Tensor vfirst, OptTensor lam, int64_t mix, int64_t v_off, int64_t v_cols) {
@@ -847,6 +876,7 @@ TORCH_LIBRARY(dlia, m) {
   m.def("gated_headnorm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, int heads, int dv, float eps) -> ()");
   m.def("gated_gelu(Tensor(a!) act, Tensor gu) -> ()");
   m.def("paged_attention_window(Tensor(a!) out, Tensor qkv, Tensor kv_cache, Tensor q_start, Tensor ctx_lens, Tensor block_table, Tensor? slots, Tensor? partial, int max_q_len, int Hq, int Hkv, int D, float scale, int splits, int window, bool sink) -> ()");
+  m.def("paged_attention_biased(Tensor(a!) out, Tensor qkv, Tensor kv_cache, Tensor q_start, Tensor ctx_lens, Tensor block_table, Tensor? slots, int max_q_len, int Hq, int Hkv, int D, float scale, Tensor? temp, Tensor? bias, Tensor? sinkv, Tensor? gate) -> ()");
   m.def("value_mix(Tensor(a!) qkv, Tensor(b!) vfirst, Tensor? lam, int mix, int v_off, int v_cols) -> ()");
   m.def("gemm_any(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, int epi) -> ()");
   m.def("kv_store(Tensor qkv, Tensor(a!)? vfirst, Tensor? lam, int mix, Tensor(b!) kcache, Tensor(c!) vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int G, int d, int dv, int q_cols) -> ()");
@@ -886,6 +916,7 @@ TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
   m.impl("gemm_any", &gemm_any);
   m.impl("gated_gelu", &gated_gelu);
   m.impl("paged_attention_window", &paged_attention_window);
+  m.impl("paged_attention_biased", &paged_attention_biased);
   m.impl("value_mix", &value_mix);
   m.impl("kv_store", &kv_store);
   m.impl("window_attention", &window_attention);

@@ -85,7 +85,11 @@ void dlia_paged_attention(void* out, const void* qkv, const void* kv_cache, cons
                           const int* q_start, const int* ctx_lens, const int* block_table,
                           const int* slots, float* partial, int B, int max_q_len, int Hq,
                           int Hkv, int D, int table_rows, int max_blocks, int num_blocks,
-                          long ldq, long ldo, float scale, int splits, hipStream_t stream, int window = 0, int sink = 0);
+                          long ldq, long ldo, float scale, int splits, hipStream_t stream, int window = 0, int sink = 0,
+                          const float* temp = nullptr, const float* bias = nullptr, int bias_rows = 0, const float* sinkv = nullptr,
+                          const float* gate = nullptr, long ldg = 0);
+// temp / bias / sinkv / gate (bf16 cache, sink set): a learned factor per head on the scores, a bias per (distance, head) and
+// the sink's score, both divided by `scale` by the caller, and a sigmoid gate logit per (token, head) on the head's output
 // (window > 0: a query at i sees the keys j with 0 <= i - j < window; sink: one more softmax term exp(0) without a value;
 // both for the bf16 cache only)
 long dlia_paged_attention_ws_floats(int B, int max_q_len, int Hq, int Hkv, int D, int splits);

@@ -109,7 +109,7 @@ def oracle_logits(cfg: dict, W, tokens: List[int]):
 
 # Stacks that differ in what a config can say: order of the layers, which stretch repeats and how often (or none), layers
 # without a feed-forward, dense and routed feed-forwards on either mixer, head counts and groupings, key / value sizes (equal,
-# unequal, not powers of two), bias tables of several sizes and reaches, expert counts, group counts of 1 and of one expert
+# unequal, not powers of two; 64 and 128, which the MFMA attention kernels take in bf16), bias tables of several sizes and reaches, expert counts, group counts of 1 and of one expert
 # each, a single chosen expert, decay ranks, widths that are no multiple of 8 and widths the packed-weight GEMMs take.
 STACKS = {
     "loop_mid": make_config([par_layer(4, 2, 16, 16, 2, 16, 24, dense(48)), gd_layer(2, 32, moe(6, 2, 24, 3, 2, 1.5)),
@@ -125,4 +125,7 @@ STACKS = {
     # sizes the packed-weight GEMMs take in bf16 (inner sizes that are multiples of 128)
     "packed": make_config([gd_layer(2, 64, moe(8, 2, 128, 2, 1, 2.0), rank=16), par_layer(4, 2, 32, 32, 2, 64, 64, dense(256), rows=20, bias_max=300),
                            par_layer(8, 1, 16, 16, 1, 128, 128, moe(4, 2, 128, 2, 2, 1.0))], vocab=96, width=128, loop=(0, 2, 2)),
+    "mfma_heads": make_config([par_layer(4, 2, 64, 64, 2, 64, 64, dense(128), rows=14, bias_max=100), gd_layer(2, 64, None, rank=16),
+                               par_layer(8, 1, 128, 128, 1, 32, 48, moe(6, 2, 64, 3, 2, 1.5), scale=0.05, rows=24, bias_max=90)],
+                              vocab=80, width=128, loop=(0, 3, 2)),
 }

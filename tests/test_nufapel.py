@@ -69,7 +69,7 @@ def test_whole_prompt(models, stack, backend, dtype):
 
 
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
-@pytest.mark.parametrize("stack", ["loop_mid", "no_loop", "packed"])
+@pytest.mark.parametrize("stack", ["loop_mid", "no_loop", "packed", "mfma_heads"])
 def test_prefill_then_long_decoding(models, stack, backend, dtype):
     """A prompt, then one token a step over several cache blocks and past every edge of the bias tables."""
     cfg, W, path = models[stack]
@@ -94,7 +94,7 @@ def test_first_tokens_alone(models, stack, backend, dtype):
 
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
 @pytest.mark.parametrize("stack,cuts", [("loop_mid", [2, 2, 3, 1, 29, 2, 31, 33, 2, 1, 5]), ("no_loop", [31, 2, 2, 36, 1, 3, 2, 17]),
-                                        ("once", [1, 2, 30, 3, 16, 17, 2, 9]), ("packed", [2, 31, 2, 1, 60, 3, 18, 2, 33])])
+                                        ("once", [1, 2, 30, 3, 16, 17, 2, 9]), ("packed", [2, 31, 2, 1, 60, 3, 18, 2, 33]), ("mfma_heads", [2, 31, 2, 1, 97, 3, 130, 2, 33])])
 def test_portions(models, stack, cuts, backend, dtype):
     """Prompts cut into portions of changing size, down to two tokens, across block edges and the recurrences' chunk edges."""
     cfg, W, path = models[stack]
@@ -106,7 +106,7 @@ def test_portions(models, stack, cuts, backend, dtype):
 
 
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
-@pytest.mark.parametrize("stack", ["loop_mid", "no_loop", "packed"])
+@pytest.mark.parametrize("stack", ["loop_mid", "no_loop", "packed", "mfma_heads"])
 def test_mixed_batches_and_reuse(models, stack, backend, dtype):
     """Unequal requests share steps (portions beside single tokens), more requests than slots over time, a pool that only holds
     the live ones: slots and blocks change hands. Every request must come out as if it ran alone."""
@@ -136,15 +136,16 @@ def test_slot_taken_over_starts_clean(models, backend, dtype):
     check(got["a"], oracle_logits(cfg, W, a), dtype, "first", alone(path, backend, dtype, a))
 
 
+@pytest.mark.parametrize("d", [16, 64])
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
-def test_far_keys_bucket_edges_and_sink(tmp_path, backend, dtype):
+def test_far_keys_bucket_edges_and_sink(tmp_path, backend, dtype, d):
     """A parallel layer whose attention weights are shaped so that one far key stands out: token 7's key is large along one
     direction, token 9 asks along it, nobody else does. The bias table is steep, so a distance that lands in the neighbouring
     row, a key that is lost, or a sink that is left out moves the asked position's logits by far more than the tolerance. The
     beacon sits at every edge of the table's rows (the linear rows, the first logarithmic ones, the last row's start), hundreds
     of tokens back across cache blocks; in a prompt, in portions and in decoding."""
     rows, far = 12, 96
-    cfg = make_config([par_layer(2, 1, 16, 16, 1, 8, 8, None, scale=1.0, rows=rows, bias_max=far)], vocab=40, width=32)
+    cfg = make_config([par_layer(2, 1, d, d, 1, 8, 8, None, scale=1.0, rows=rows, bias_max=far)], vocab=40, width=32)
     W = random_weights(cfg, seed=5)
     for n in ("l0.mix.left.q", "l0.mix.left.k"):
         W[n] = torch.zeros_like(W[n])
@@ -154,7 +155,7 @@ def test_far_keys_bucket_edges_and_sink(tmp_path, backend, dtype):
     h9 = O.dyt(W["embed"][9].double(), W["l0.norm1"].double(), W["l0.norm1.b"].double(), W["l0.norm1.alpha"].double())
     W["l0.mix.left.k"][0] = (h7 * 0.6).to(torch.bfloat16)
     W["l0.mix.left.q"][0] = (h9 * 0.6).to(torch.bfloat16)
-    W["l0.mix.left.q"][16] = (h9 * 0.6).to(torch.bfloat16)
+    W["l0.mix.left.q"][d] = (h9 * 0.6).to(torch.bfloat16)
     W["l0.mix.left.rel"] = (torch.arange(rows).float().view(-1, 1) * torch.tensor([[1.5, -1.5]])).to(torch.bfloat16)
     W["l0.mix.left.sink"] = torch.tensor([24.0, 7.0], dtype=torch.bfloat16)
     path = save(str(tmp_path / "m"), cfg, W)
@@ -182,7 +183,7 @@ def test_far_keys_bucket_edges_and_sink(tmp_path, backend, dtype):
     assert rel_err(at(toks, W), at(moved, W)) > 0.02 and rel_err(at(toks, W), at(none, W)) > 0.02 and rel_err(at(toks, W), at(toks, nosink)) > 0.02
 
 
-@pytest.mark.parametrize("stack,buckets", [("loop_mid", []), ("packed", []), ("no_loop", [2])])
+@pytest.mark.parametrize("stack,buckets", [("loop_mid", []), ("packed", []), ("no_loop", [2]), ("mfma_heads", [])])
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
 def test_greedy_generation_through_the_scheduler(models, backend, dtype, stack, buckets):
     """Requests of unequal length through the engine's own entry point: scheduler, continuous batching, chunked prompts, greedy
