@@ -31,6 +31,22 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Sum over the R adjacent lanes that share a value column (R a power of two up to 16), every lane ending with the
+// total: data-parallel-primitive moves inside the quad, the half row and the row — no LDS round trip, which a
+// ds_bpermute shuffle is, twice per token on the recurrence's critical path.
+template <int CTRL>
+__device__ __forceinline__ float dpp_term(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+template <int R>
+__device__ __forceinline__ float group_sum(float x) {
+  if constexpr (R >= 2) x += dpp_term<0xB1>(x);      // quad_perm [1, 0, 3, 2]
+  if constexpr (R >= 4) x += dpp_term<0x4E>(x);      // quad_perm [2, 3, 0, 1]
+  if constexpr (R >= 8) x += dpp_term<0x141>(x);     // row_half_mirror: the other quad of the 8 lanes holds its own sum
+  if constexpr (R >= 16) x += dpp_term<0x140>(x);    // row_mirror: the other half of the 16 lanes
+  return x;
+}
+
 // Block reductions through LDS; `scratch` must hold >= 16 floats. blockDim.x multiple of 64.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
   v = wave_sum(v);

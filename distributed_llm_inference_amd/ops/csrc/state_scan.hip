@@ -17,6 +17,7 @@
 // owns state slot slots[b]; ctx 0 starts from zeros (m from 0) whatever the slot held, so slots change hands without clearing.
 // The running maximum is kept once per column block (mstate [slots, H, kScanMaxBlocks]), so that no workgroup reads what
 // another one writes.
+#include <stdlib.h>
 #include "common.h"
 #include "launch.h"
 
@@ -42,7 +43,7 @@ __device__ __forceinline__ float logsigmoidf_(float x) { return x >= 0.f ? -log1
 
 template <int RULE>
 __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int NV = RULE == 0 ? 5 : 2;
   const int b = blockIdx.x, h = blockIdx.y, zb = blockIdx.z;
   const int t0 = p.q_start[b], n = p.q_start[b + 1] - t0, c0 = p.ctx[b], slot = p.slots[b];
@@ -163,6 +164,178 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
   if (RULE == 1 && tid == 0) mp[0] = m_run;
 }
 
+// The same walk for key sizes up to 128 with everything that sits on the chain from one token to the next made short. A
+// workgroup's four waves each sit alone on a SIMD, so nothing hides latency: the time per token IS the dependent chain. Here
+// a column's rows are spread over R <= 8 lanes known at compile time (16 rows each; in LDS every 16 rows are followed by 4 words
+// of padding, so that the 16-byte reads of lanes with different rows fall into different banks: without it the reads of a wave
+// collide four ways and the LDS pipe, not the arithmetic, sets the time per token), the two sums over the rows run as four
+// independent chains and finish with data-parallel-primitive moves between neighbouring lanes (no LDS round trip), the NEXT
+// chunk's inputs are fetched into registers before the current chunk is walked and become LDS contents (gates evaluated, key
+// normalised) after it. Rule 1's running maximum is a prefix scan over the chunk's tokens in the (max, +) algebra —
+// m -> max(a + m, b) composes as (a1 + a2, max(a2 + b1, b2)) — done by the first 16 lanes of every wave with shuffles, so it
+// costs no barrier and no serial loop; the per-token factors then travel by lane broadcast.
+constexpr int kFastRows = 16, kFastPad = 4;
+
+template <int RULE, int R>
+__global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr int NV = RULE == 0 ? 5 : 2, CB = 256 / R, DP = (kFastRows + kFastPad) * R, CH = 16, VPL = CB / 16, EL = R;
+  auto at = [](int row) { return row + (row / kFastRows) * kFastPad; };      // a row's place in a padded vector
+  const int b = blockIdx.x, h = blockIdx.y, zb = blockIdx.z;
+  const int t0 = p.q_start[b], n = p.q_start[b + 1] - t0, c0 = p.ctx[b], slot = p.slots[b];
+  if (n <= 0 || slot < 0 || slot >= p.state_rows) return;
+  const int tid = threadIdx.x, d = p.d, NC = p.NC;
+  const int c = tid / R, rg = tid % R, j = zb * CB + c;
+  const bool col_ok = j < NC;
+  float* vec = lds;                                  // [CH][NV][DP]
+  float* vals = vec + CH * NV * DP;                  // [CH][CB]
+  float* sc = vals + CH * CB;                        // [CH][2]: rule 1: log i, log f
+  float* S = p.state + ((long)slot * p.H + h) * (long)d * NC;
+  float s[kFastRows];
+#pragma unroll
+  for (int e = 0; e < kFastRows; ++e) {
+    const int row = rg * kFastRows + e;
+    s[e] = (c0 > 0 && col_ok && row < d) ? S[(long)row * NC + j] : 0.f;
+  }
+  float* mp = p.mstate ? p.mstate + ((long)slot * p.H + h) * kScanMaxBlocks + zb : nullptr;
+  float m_run = 0.f;
+  if constexpr (RULE == 1) m_run = c0 > 0 ? mp[0] : 0.f;
+  const int tt = tid >> 4, sub = tid & 15, hd = h * d, lane = tid & 63;
+  float pa[EL], pb[EL], pc[RULE == 0 ? EL : 1], pd[RULE == 0 ? EL : 1], pv[VPL], pi = 0.f, pf = 0.f;
+
+  auto prefetch = [&](int ch0) {
+    if (tt >= min(CH, n - ch0)) return;
+    const long t = t0 + ch0 + tt;
+    const float* zr = p.z + t * p.ldz;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const int i = sub * EL + e;
+      const bool ok = i < d;
+      pa[e] = ok ? zr[p.col_k + hd + i] : 0.f;
+      pb[e] = ok ? zr[p.col_q + hd + i] : 0.f;
+      if constexpr (RULE == 0) {
+        pc[e] = ok ? zr[p.col_a + hd + i] + p.b0[hd + i] : 0.f;
+        pd[e] = ok ? p.wz[t * p.ldw + hd + i] + p.b1[hd + i] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) {
+      const int jj = zb * CB + sub * VPL + e;
+      pv[e] = jj < p.dv ? zr[p.col_v + h * p.dv + jj] : ((RULE == 1 && jj == p.dv) ? 1.f : 0.f);
+    }
+    if constexpr (RULE == 1) {
+      if (sub == 0) { pi = zr[p.col_i + h] + p.b0[h]; pf = zr[p.col_f + h] + p.b0[p.H + h]; }
+    }
+  };
+  auto commit = [&](int nt) {
+    if (tt >= nt) return;
+    float* vt = vec + tt * NV * DP;
+    if constexpr (RULE == 0) {
+      float ksq = 0.f;
+#pragma unroll
+      for (int e = 0; e < EL; ++e) ksq += pa[e] * pa[e];
+      ksq = group_sum<16>(ksq);
+      const float inv = rsqrtf(ksq + 1e-6f);
+#pragma unroll
+      for (int e = 0; e < EL; ++e) {
+        const bool ok = sub * EL + e < d;
+        const float u = pa[e] * inv;
+        float* v0 = vt + at(sub * EL + e);
+        v0[0] = ok ? expf(-0.6065306597126334f * sigmoidf_(pd[e])) : 0.f;
+        v0[DP] = ok ? sigmoidf_(pc[e]) * u : 0.f;
+        v0[2 * DP] = u; v0[3 * DP] = pa[e]; v0[4 * DP] = pb[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EL; ++e) { float* v0 = vt + at(sub * EL + e); v0[0] = pa[e]; v0[DP] = pb[e] * p.qscale; }
+      if (sub == 0) {
+        sc[tt * 2] = p.cap * tanhf(pi / p.cap);
+        sc[tt * 2 + 1] = logsigmoidf_(p.cap * tanhf(pf / p.cap));
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) vals[tt * CB + sub * VPL + e] = pv[e];
+  };
+
+  prefetch(0);
+  for (int ch0 = 0; ch0 < n; ch0 += CH) {
+    const int nt = min(CH, n - ch0);
+    __syncthreads();                                 // the previous chunk has been walked
+    commit(nt);
+    __syncthreads();
+    if (ch0 + CH < n) prefetch(ch0 + CH);            // in flight while this chunk is walked
+    [[maybe_unused]] float keepv = 1.f, putv = 0.f, emv = 1.f;
+    if constexpr (RULE == 1) {
+      const bool live = lane < nt;
+      const float lf = live ? sc[(lane & 15) * 2 + 1] : 0.f, li = live ? sc[(lane & 15) * 2] : -INFINITY;
+      float a = lf, bb = li;                         // the token's own map m -> max(a + m, b); lanes past the chunk: the identity
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) {
+        const float ea = __shfl_up(a, o, 64), eb = __shfl_up(bb, o, 64);
+        if ((lane & 15) >= o) { bb = fmaxf(a + eb, bb); a = ea + a; }
+      }
+      const float m_t = fmaxf(a + m_run, bb);
+      float m_prev = __shfl_up(m_t, 1, 64);
+      if ((lane & 15) == 0) m_prev = m_run;
+      keepv = expf(lf + m_prev - m_t); putv = expf(li - m_t); emv = expf(-m_t);
+      m_run = __shfl(m_t, nt - 1, 64);
+    }
+    for (int q = 0; q < nt; ++q) {
+      const float* v0 = vec + q * NV * DP + rg * (kFastRows + kFastPad);
+      const float v = vals[q * CB + c];
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (RULE == 0) {
+        float d4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < kFastRows; ++e) d4[e & 3] += v0[2 * DP + e] * s[e];
+        const float dot = group_sum<R>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+#pragma unroll
+        for (int e = 0; e < kFastRows; ++e) {
+          s[e] = v0[e] * s[e] - v0[DP + e] * dot + v0[3 * DP + e] * v;
+          o4[e & 3] += v0[4 * DP + e] * s[e];
+        }
+      } else {
+        const float keep = __shfl(keepv, q, 64), put = __shfl(putv, q, 64) * v;
+#pragma unroll
+        for (int e = 0; e < kFastRows; ++e) {
+          s[e] = keep * s[e] + put * v0[e];
+          o4[e & 3] += v0[DP + e] * s[e];
+        }
+      }
+      const float out = group_sum<R>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      [[maybe_unused]] const float em = RULE == 1 ? __shfl(emv, q, 64) : 0.f;
+      if (rg == 0 && col_ok) {
+        float* orow = p.o + (long)(t0 + ch0 + q) * p.ldo;
+        if constexpr (RULE == 0) orow[h * p.dv + j] = out;
+        else {
+          orow[h * (p.dv + 2) + j] = out;
+          if (j == p.dv) orow[h * (p.dv + 2) + p.dv + 1] = em;
+        }
+      }
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int e = 0; e < kFastRows; ++e) {
+      const int row = rg * kFastRows + e;
+      if (row < d) S[(long)row * NC + j] = s[e];
+    }
+  }
+  if constexpr (RULE == 1) {
+    if (tid == 0) mp[0] = m_run;
+  }
+}
+
+template <int RULE>
+static void launch_scan_fast(const ScanArgs& p, int R, dim3 grid, hipStream_t stream) {
+  const int nv = RULE == 0 ? 5 : 2;
+  const size_t lds = (size_t)16 * (nv * (kFastRows + kFastPad) * R + 256 / R + 2) * sizeof(float);
+  if (R == 1) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 1>), grid, dim3(256), lds, stream, p);
+  else if (R == 2) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 2>), grid, dim3(256), lds, stream, p);
+  else if (R == 4) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 4>), grid, dim3(256), lds, stream, p);
+  else hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 8>), grid, dim3(256), lds, stream, p);
+}
+
 }  // namespace dlia
 
 // Column blocks a (d, columns) state is split into: the launch shape depends on the sizes only, never on the step.
@@ -195,6 +368,14 @@ extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, lon
   if (ZB > dlia::kScanMaxBlocks) return 2;
   const size_t lds = (size_t)p.CH * per_token * sizeof(float);
   const dim3 grid(B, H, ZB);
+  static const bool fast_on = [] { const char* e = getenv("DLIA_SCAN_FAST"); return !(e && atoi(e) == 0); }();
+  if (d <= 8 * dlia::kFastRows && fast_on) {
+    int Rf = 1;
+    while (Rf * dlia::kFastRows < d) Rf <<= 1;
+    const dim3 gridf(B, H, (p.NC + 256 / Rf - 1) / (256 / Rf));
+    if (rule == 0) dlia::launch_scan_fast<0>(p, Rf, gridf, stream); else dlia::launch_scan_fast<1>(p, Rf, gridf, stream);
+    return 0;
+  }
   if (rule == 0)
     hipLaunchKernelGGL(dlia::state_scan_kernel<0>, grid, dim3(256), lds, stream, p);
   else
