@@ -280,37 +280,57 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
       keepv = expf(lf + m_prev - m_t); putv = expf(li - m_t); emv = expf(-m_t);
       m_run = __shfl(m_t, nt - 1, 64);
     }
-    for (int q = 0; q < nt; ++q) {
+    // two register sets: the vectors of token q + 1 are read from LDS while token q is applied
+    float va[NV][kFastRows], vb[NV][kFastRows], xa, xb = 0.f;
+    auto fetch = [&](float (&dst)[NV][kFastRows], float& x, int q) {
       const float* v0 = vec + q * NV * DP + rg * (kFastRows + kFastPad);
-      const float v = vals[q * CB + c];
+#pragma unroll
+      for (int k = 0; k < NV; ++k)
+#pragma unroll
+        for (int e = 0; e < kFastRows; e += 4) {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(v0 + k * DP + e);
+          dst[k][e] = t.x; dst[k][e + 1] = t.y; dst[k][e + 2] = t.z; dst[k][e + 3] = t.w;
+        }
+      x = vals[q * CB + c];
+    };
+    auto apply = [&](const float (&w)[NV][kFastRows], float v, int q) {
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
       if constexpr (RULE == 0) {
         float d4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int e = 0; e < kFastRows; ++e) d4[e & 3] += v0[2 * DP + e] * s[e];
+        for (int e = 0; e < kFastRows; ++e) d4[e & 3] += w[2][e] * s[e];
         const float dot = group_sum<R>((d4[0] + d4[1]) + (d4[2] + d4[3]));
 #pragma unroll
         for (int e = 0; e < kFastRows; ++e) {
-          s[e] = v0[e] * s[e] - v0[DP + e] * dot + v0[3 * DP + e] * v;
-          o4[e & 3] += v0[4 * DP + e] * s[e];
+          s[e] = w[0][e] * s[e] - w[1][e] * dot + w[3][e] * v;
+          o4[e & 3] += w[4][e] * s[e];
         }
       } else {
-        const float keep = __shfl(keepv, q, 64), put = __shfl(putv, q, 64) * v;
+        const float keep = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, keepv), q));
+        const float put = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, putv), q)) * v;
 #pragma unroll
         for (int e = 0; e < kFastRows; ++e) {
-          s[e] = keep * s[e] + put * v0[e];
-          o4[e & 3] += v0[DP + e] * s[e];
+          s[e] = keep * s[e] + put * w[0][e];
+          o4[e & 3] += w[1][e] * s[e];
         }
       }
       const float out = group_sum<R>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-      [[maybe_unused]] const float em = RULE == 1 ? __shfl(emv, q, 64) : 0.f;
       if (rg == 0 && col_ok) {
         float* orow = p.o + (long)(t0 + ch0 + q) * p.ldo;
         if constexpr (RULE == 0) orow[h * p.dv + j] = out;
         else {
           orow[h * (p.dv + 2) + j] = out;
-          if (j == p.dv) orow[h * (p.dv + 2) + p.dv + 1] = em;
+          if (j == p.dv) orow[h * (p.dv + 2) + p.dv + 1] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, emv), q));
         }
+      }
+    };
+    fetch(va, xa, 0);
+    for (int q = 0; q < nt; q += 2) {
+      if (q + 1 < nt) fetch(vb, xb, q + 1);
+      apply(va, xa, q);
+      if (q + 1 < nt) {
+        if (q + 2 < nt) fetch(va, xa, q + 2);
+        apply(vb, xb, q + 1);
       }
     }
   }
@@ -350,7 +370,7 @@ extern "C" int dlia_state_scan_blocks(int d, int ncols) {
 extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, const float* wz, long ldw, float* state,
                                float* mstate, const float* b0, const float* b1, const int* q_start, const int* ctx,
                                const int* slots, int B, int H, int d, int dv, int state_rows, int col_q, int col_k, int col_v,
-                               int col_a, int col_i, int col_f, float cap, float qscale, hipStream_t stream) {
+                               int col_a, int col_i, int col_f, float cap, float qscale, int max_q, hipStream_t stream) {
   if (B <= 0) return 0;
   dlia::ScanArgs p;
   p.o = o; p.ldo = ldo; p.z = z; p.ldz = ldz; p.wz = wz; p.ldw = ldw; p.state = state; p.mstate = mstate; p.b0 = b0; p.b1 = b1;
@@ -369,7 +389,9 @@ extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, lon
   const size_t lds = (size_t)p.CH * per_token * sizeof(float);
   const dim3 grid(B, H, ZB);
   static const bool fast_on = [] { const char* e = getenv("DLIA_SCAN_FAST"); return !(e && atoi(e) == 0); }();
-  if (d <= 8 * dlia::kFastRows && fast_on) {
+  // (steps of few tokens per sequence — decoding — run many workgroups at once: there the kernel that needs a third of the
+  // registers keeps more of them resident, and there is no chain of tokens to shorten)
+  if (d <= 8 * dlia::kFastRows && fast_on && max_q >= 8) {
     int Rf = 1;
     while (Rf * dlia::kFastRows < d) Rf <<= 1;
     const dim3 gridf(B, H, (p.NC + 256 / Rf - 1) / (256 / Rf));

@@ -95,7 +95,7 @@ def test_general_delta_rule_hip(H, d):
         o = torch.zeros(z.shape[0], n, device="cuda")
         q0, c, s = _meta(ql, cx, sl)
         # (the three sequences share w0 / a.b here: one layer's vectors)
-        K.state_scan(0, o, z, wz, state, None, _dev(t0["x.a.b"]), _dev(t0["x.w0"]), q0, c, s, H, d, d, 0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0)
+        K.state_scan(0, o, z, wz, state, None, _dev(t0["x.a.b"]), _dev(t0["x.w0"]), q0, c, s, H, d, d, 0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0, max(ql))
         mixed = torch.zeros(z.shape[0], n, device="cuda")
         K.headnorm_gate(mixed, o, z[:, 3 * n:4 * n], _dev(t0["x.norm"]), H, d, 0, 1e-5)
         at = 0
@@ -157,7 +157,7 @@ def test_matrix_memory_hip(H, d, dv, cap):
         o = torch.zeros(z.shape[0], H * (dv + 2), device="cuda")
         q0, c, s = _meta(ql, cx, sl)
         K.state_scan(1, o, z, None, state, mstate, _dev(torch.cat([t0["x.i.b"], t0["x.f.b"]])), None, q0, c, s, H, d, dv,
-                     int(cq), int(ck), int(cv), 0, int(ci), int(cf), cap, d ** -0.5)
+                     int(cq), int(ck), int(cv), 0, int(ci), int(cf), cap, d ** -0.5, max(ql))
         mixed = torch.zeros(z.shape[0], H * dv, device="cuda")
         K.headnorm_gate(mixed, o, z[:, int(cg):int(cg) + H * dv], _dev(t0["x.norm"]), H, dv, 2, 1e-5)
         at = 0
