@@ -469,7 +469,7 @@ class HybridGpuStage(GpuStage):
                 z2 = max(z2, self._cols(p, "w_ff"))
                 if ls.moe is not None:
                     e = ls.moe
-                    pairs, tiles, ef = max(pairs, rows * e.top), max(tiles, (rows * e.top + 15) // 16 + e.experts), max(ef, e.ff)
+                    pairs, tiles, ef = max(pairs, rows * e.top), max(tiles, (rows * e.top + 31) // 32 + e.experts), max(ef, e.ff)
                 else:
                     ac, yc = max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
         ws_floats = self._ws_floats
@@ -482,7 +482,7 @@ class HybridGpuStage(GpuStage):
             h=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), wz=z(rows * wc),
             low=z(rows * lc, at), o=z(rows * oc), mixed=z(rows * mc, at), mixed2=z(rows * m2, at), ya=z(rows * yc), yb=z(rows * yc),
             z2=z(rows * z2), act=z(rows * ac, at), sel=z(pairs, i32), wts=z(pairs), pair_row=z(pairs, i32), tiles=z(1 + tiles, i32),
-            row_tok=z(16 * tiles, i32), eact=z(16 * tiles * ef, at), ey=z(16 * tiles * H), ws=z(ws_floats + 4096),
+            row_tok=z(32 * tiles, i32), eact=z(32 * tiles * ef, at), ey=z(32 * tiles * H), ws=z(ws_floats + 4096),
             qkv16=z(rows * qc, torch.bfloat16),
             head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
 
@@ -569,8 +569,8 @@ class HybridGpuStage(GpuStage):
                     g0 = ls.ff
                 else:
                     e = ls.moe
-                    nt = (T * e.top + 15) // 16 + e.experts
-                    eact, ey, ya = wk.eact[:16 * nt * e.ff].view(16 * nt, e.ff), wk.ey[:16 * nt * H].view(16 * nt, H), view(wk.ya, H)
+                    nt = (T * e.top + 31) // 32 + e.experts          # row tiles of 32: at most this many hold a row
+                    eact, ey, ya = wk.eact[:32 * nt * e.ff].view(32 * nt, e.ff), wk.ey[:32 * nt * H].view(32 * nt, H), view(wk.ya, H)
                     K.moe_route(wk.sel, wk.wts, z2[:, :e.experts], e.top, e.groups, e.keep, e.scale)
                     K.moe_plan(wk.tiles, wk.row_tok, wk.pair_row, wk.sel, T * e.top, e.top, e.experts)
                     K.moe_up(eact, xn, p["w_gate_e"], p["w_up_e"], wk.tiles, wk.row_tok, nt, e.limit)

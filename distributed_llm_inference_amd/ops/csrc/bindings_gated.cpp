@@ -216,11 +216,11 @@ void moe_route(Tensor sel, Tensor wts, const Tensor& logits, int64_t top, int64_
 void moe_plan(Tensor tiles, Tensor row_tok, Tensor pair_row, const Tensor& sel, int64_t pairs, int64_t top, int64_t E) {
   DLIA_ON_DEVICE_OF(tiles);
   check_i32(tiles, "tiles"); check_i32(row_tok, "row_tok"); check_i32(pair_row, "pair_row"); check_i32(sel, "sel");
-  const int64_t max_tiles = (pairs + 15) / 16 + E;
+  const int64_t max_tiles = (pairs + 31) / 32 + E;
   DLIA_CHECK(E >= 1 && E <= 256 && top >= 1 && pairs >= 0 && sel.numel() >= pairs && pair_row.numel() >= pairs, "moe_plan: pairs");
-  DLIA_CHECK(tiles.numel() >= 1 + max_tiles && row_tok.numel() >= 16 * max_tiles, "moe_plan: room for pairs / 16 + E tiles");
+  DLIA_CHECK(tiles.numel() >= 1 + max_tiles && row_tok.numel() >= 32 * max_tiles, "moe_plan: room for pairs / 32 + E tiles of 32 rows");
   dlia_moe_plan(tiles.data_ptr<int>(), row_tok.data_ptr<int>(), pair_row.data_ptr<int>(), sel.data_ptr<int>(), (int)pairs, (int)top, (int)E,
-                (int)(16 * max_tiles), cur_stream());
+                (int)(32 * max_tiles), cur_stream());
 }
 
 void moe_up(Tensor act, const Tensor& x, const Tensor& wg, const Tensor& wu, const Tensor& tiles, const Tensor& row_tok, int64_t max_tiles,
@@ -231,20 +231,20 @@ void moe_up(Tensor act, const Tensor& x, const Tensor& wg, const Tensor& wu, con
   DLIA_CHECK(wg.dim() == 3 && wg.is_contiguous() && wu.is_contiguous() && wu.sizes() == wg.sizes() && wg.size(2) == x.size(1) &&
              x.scalar_type() == wg.scalar_type() && wu.scalar_type() == wg.scalar_type() && act.scalar_type() == x.scalar_type(),
              "moe_up: x [T, K], wg / wu [E, F, K], one type");
-  DLIA_CHECK(act.size(1) == wg.size(1) && act.size(0) >= 16 * max_tiles && row_tok.numel() >= 16 * max_tiles && tiles.numel() >= 1 + max_tiles,
-             "moe_up: act [16 max_tiles, F]");
+  DLIA_CHECK(act.size(1) == wg.size(1) && act.size(0) >= 32 * max_tiles && row_tok.numel() >= 32 * max_tiles && tiles.numel() >= 1 + max_tiles,
+             "moe_up: act [32 max_tiles, F]");
   dlia_moe_up(act.data_ptr(), x.data_ptr(), wg.data_ptr(), wu.data_ptr(), is_f32(x), tiles.data_ptr<int>(), row_tok.data_ptr<int>(),
-              (int)max_tiles, (int)wg.size(1), (int)wg.size(2), x.stride(0), act.stride(0), (float)limit, cur_stream());
+              (int)max_tiles, x.size(0) > 256 ? 1 : 0, (int)wg.size(1), (int)wg.size(2), x.stride(0), act.stride(0), (float)limit, cur_stream());
 }
 
 void moe_down(Tensor y, const Tensor& act, const Tensor& wd, const Tensor& tiles, const Tensor& row_tok, int64_t max_tiles) {
   DLIA_ON_DEVICE_OF(y);
   check_f32(y, "y"); check_act(act, "act"); check_mat(act, "act"); check_act(wd, "wd"); check_i32(tiles, "tiles"); check_i32(row_tok, "row_tok");
   DLIA_CHECK(wd.dim() == 3 && wd.is_contiguous() && wd.size(2) == act.size(1) && wd.scalar_type() == act.scalar_type(), "moe_down: wd [E, H, F]");
-  DLIA_CHECK(y.dim() == 2 && y.size(1) == wd.size(1) && y.size(0) >= 16 * max_tiles && act.size(0) >= 16 * max_tiles &&
-             row_tok.numel() >= 16 * max_tiles && tiles.numel() >= 1 + max_tiles, "moe_down: y [16 max_tiles, H]");
+  DLIA_CHECK(y.dim() == 2 && y.size(1) == wd.size(1) && y.size(0) >= 32 * max_tiles && act.size(0) >= 32 * max_tiles &&
+             row_tok.numel() >= 32 * max_tiles && tiles.numel() >= 1 + max_tiles, "moe_down: y [32 max_tiles, H]");
   dlia_moe_down(y.data_ptr<float>(), act.data_ptr(), wd.data_ptr(), is_f32(act), tiles.data_ptr<int>(), row_tok.data_ptr<int>(),
-                (int)max_tiles, (int)wd.size(1), (int)wd.size(2), act.stride(0), cur_stream());
+                (int)max_tiles, max_tiles > 64 ? 1 : 0, (int)wd.size(1), (int)wd.size(2), act.stride(0), cur_stream());
 }
 
 void moe_combine(Tensor out, const Tensor& y, const Tensor& pair_row, const Tensor& wts, int64_t top) {

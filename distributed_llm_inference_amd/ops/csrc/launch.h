@@ -167,9 +167,10 @@ void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, i
 void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows,
                    hipStream_t stream);
 void dlia_moe_up(void* act, const void* x, const void* wg, const void* wu, int f32, const int* tiles, const int* row_tok,
-                 int max_tiles, int F, int K, long ldx, long lda, float limit, hipStream_t stream);
-void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok, int max_tiles, int H,
-                   int F, long lda, hipStream_t stream);
+                 int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, hipStream_t stream);
+void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok, int max_tiles, int wide,
+                   int H, int F, long lda, hipStream_t stream);
+// (wide: 128 / 256 output columns per workgroup, for steps with many rows; else 64)
 void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
                       hipStream_t stream);
 

@@ -1,16 +1,15 @@
 // Routed feed-forward (mixture of experts) without a host round trip: routing, a plan that sorts the step's (token, choice)
-// pairs by expert into 16-row tiles, the experts' two GEMMs over those tiles, and the weighted sum per token.
+// pairs by expert into 32-row tiles, the experts' two GEMMs over those tiles, and the weighted sum per token.
 //
 //   moe_route    one thread per token. Scores are sigmoids of the fp32 router logits. Experts form `groups` equal groups of
 //                neighbours; a group's score is the sum of its two largest scores; the `keep` best groups stay; the `top`
 //                best experts of those are chosen (equal scores: the lower index), weighted score / (sum + 1e-20) * scale.
 //   moe_plan     one workgroup. Counts the pairs per expert, lays the experts' row ranges out one after the other, each
-//                padded to whole 16-row tiles, and writes for every padded row its token (or -1), for every pair its row,
+//                padded to whole 32-row tiles, and writes for every padded row its token (or -1), for every pair its row,
 //                for every tile its expert; tiles[0] holds the number of tiles. Rows of one expert are in no fixed order:
 //                every row is computed on its own, so the order does not reach the results.
 //   moe_up       grid (column blocks, tiles): act[row, f] = g s(1.702 g) (u + 1), g = min(x . Wg[e][f], limit),
-//                u = clamp(x . Wu[e][f], -limit, limit), x the row's token. One wave per 16 columns, gate and up in two
-//                accumulators over the same A fragments.
+//                u = clamp(x . Wu[e][f], -limit, limit), x the row's token; gate and up accumulate over the same A fragments.
 //   moe_down     y[row, c] = act[row] . Wd[e][c] in fp32.
 //   moe_combine  out[t, :] = sum over the token's choices of weight * y[row, :], in the order of the choices (fp32).
 // Operands are bf16 (16x16x32 MFMA) or fp32 (16x16x4 MFMA, true 32-bit), fragments read straight from the K-contiguous rows.
@@ -21,6 +20,7 @@
 namespace dlia {
 
 constexpr int kMoeMaxExperts = 256;
+constexpr int kMoeRows = 32;           // rows of a plan tile
 
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ sel, float* __restrict__ wts,
                                                        const float* __restrict__ logits, long ld, int T, int E, int top,
@@ -79,15 +79,15 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles,
     int at = 0, nt = 0;
     for (int e = 0; e < E; ++e) {
       start[e] = at;
-      const int n = (count[e] + 15) / 16;
+      const int n = (count[e] + kMoeRows - 1) / kMoeRows;
       for (int i = 0; i < n; ++i) tiles[1 + nt + i] = e;
-      nt += n; at += n * 16;
+      nt += n; at += n * kMoeRows;
     }
     tiles[0] = nt;
     ntiles = nt;
   }
   __syncthreads();
-  const int used = ntiles * 16;
+  const int used = ntiles * kMoeRows;
   for (int i = threadIdx.x; i < max_rows; i += 1024) row_tok[i] = -1;
   __syncthreads();
   for (int i = threadIdx.x; i < pairs; i += 1024) {
@@ -97,7 +97,12 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles,
   }
 }
 
-template <typename T, typename OT>
+// Row tiles of the plan: 32 rows. A workgroup of four waves covers one row tile by 128 (up) or 256 (down) output columns; a
+// wave holds both 16-row halves of the tile against its 32 (64) columns, so every fragment it loads feeds two or more MFMAs,
+// and the fragments of the next k-step are on their way while the current ones are multiplied.
+constexpr int kMoeTile = kMoeRows;
+
+template <typename T, typename OT, int NJ>
 __global__ __launch_bounds__(256) void moe_up_kernel(OT* __restrict__ act, const T* __restrict__ x, const T* __restrict__ wg,
                                                      const T* __restrict__ wu, const int* __restrict__ tiles,
                                                      const int* __restrict__ row_tok, int F, int K, long ldx, long lda,
@@ -107,29 +112,64 @@ __global__ __launch_bounds__(256) void moe_up_kernel(OT* __restrict__ act, const
   if (tile >= tiles[0]) return;
   const int e = tiles[1 + tile];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, kq = lane >> 4;
-  const int f0 = blockIdx.x * 64 + wave * 16;
+  const int f0 = (blockIdx.x * 4 + wave) * 16 * NJ;
   if (f0 >= F) return;
-  const int tok = row_tok[tile * 16 + r16];
-  const bool av = tok >= 0, wv = f0 + r16 < F;
-  const T* arow = x + (long)(av ? tok : 0) * ldx;
-  const long wrow = ((long)e * F + (wv ? f0 + r16 : 0)) * K;
-  f32x4 ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += KS) {
-    const int k = k0 + kq * VEC;
-    const u32x4 a = load_frag<T>(arow, k, K, av, vec_ok);
-    ag = mma_frag(T{}, a, load_frag<T>(wg + wrow, k, K, wv, vec_ok), ag);
-    au = mma_frag(T{}, a, load_frag<T>(wu + wrow, k, K, wv, vec_ok), au);
-  }
-  if (!wv) return;
+  const T* arow[2]; long wrow[NJ]; bool av[2], wv[NJ];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = tile * 16 + kq * 4 + r;
-    const float g = fminf(ag[r], limit), u = fminf(fmaxf(au[r], -limit), limit);
-    act[(long)row * lda + f0 + r16] = (OT)(g / (1.f + expf(-1.702f * g)) * (u + 1.f));
+  for (int i = 0; i < 2; ++i) {
+    const int tok = row_tok[tile * kMoeTile + i * 16 + r16];
+    av[i] = tok >= 0;
+    arow[i] = x + (long)(av[i] ? tok : 0) * ldx;
   }
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    wv[j] = f0 + j * 16 + r16 < F;
+    wrow[j] = ((long)e * F + (wv[j] ? f0 + j * 16 + r16 : 0)) * K;
+  }
+  f32x4 ag[2][NJ], au[2][NJ];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { ag[i][j] = f32x4{0.f, 0.f, 0.f, 0.f}; au[i][j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+  u32x4 a[2], g[NJ], u[NJ], an[2], gn[NJ], un[NJ];
+  auto load = [&](u32x4 (&fa)[2], u32x4 (&fg)[NJ], u32x4 (&fu)[NJ], int k0) {
+    const int k = k0 + kq * VEC;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[i] = load_frag<T>(arow[i], k, K, av[i], vec_ok);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      fg[j] = load_frag<T>(wg + wrow[j], k, K, wv[j], vec_ok);
+      fu[j] = load_frag<T>(wu + wrow[j], k, K, wv[j], vec_ok);
+    }
+  };
+  load(a, g, u, 0);
+  for (int k0 = 0; k0 < K; k0 += KS) {
+    if (k0 + KS < K) load(an, gn, un, k0 + KS);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) { ag[i][j] = mma_frag(T{}, a[i], g[j], ag[i][j]); au[i][j] = mma_frag(T{}, a[i], u[j], au[i][j]); }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a[i] = an[i];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { g[j] = gn[j]; u[j] = un[j]; }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int col = f0 + j * 16 + r16;
+      if (col >= F) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = tile * kMoeTile + i * 16 + kq * 4 + r;
+        const float gv = fminf(ag[i][j][r], limit), uv = fminf(fmaxf(au[i][j][r], -limit), limit);
+        act[(long)row * lda + col] = (OT)(gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f));
+      }
+    }
 }
 
-template <typename T>
+template <typename T, int NJ>
 __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ y, const T* __restrict__ act, const T* __restrict__ wd,
                                                        const int* __restrict__ tiles, const int* __restrict__ row_tok,
                                                        int H, int F, long lda, int vec_ok) {
@@ -138,19 +178,53 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ y, co
   if (tile >= tiles[0]) return;
   const int e = tiles[1 + tile];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, kq = lane >> 4;
-  const int c0 = blockIdx.x * 64 + wave * 16;
+  const int c0 = (blockIdx.x * 4 + wave) * 16 * NJ;
   if (c0 >= H) return;
-  const bool av = row_tok[tile * 16 + r16] >= 0, wv = c0 + r16 < H;
-  const T* arow = act + (long)(tile * 16 + r16) * lda;
-  const T* wrow = wd + ((long)e * H + (wv ? c0 + r16 : 0)) * F;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < F; k0 += KS) {
-    const int k = k0 + kq * VEC;
-    acc = mma_frag(T{}, load_frag<T>(arow, k, F, av, vec_ok), load_frag<T>(wrow, k, F, wv, vec_ok), acc);
-  }
-  if (!wv) return;
+  const T* arow[2]; const T* wrow[NJ]; bool av[2], wv[NJ];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) y[(long)(tile * 16 + kq * 4 + r) * H + c0 + r16] = acc[r];
+  for (int i = 0; i < 2; ++i) {
+    av[i] = row_tok[tile * kMoeTile + i * 16 + r16] >= 0;
+    arow[i] = act + (long)(tile * kMoeTile + i * 16 + r16) * lda;
+  }
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    wv[j] = c0 + j * 16 + r16 < H;
+    wrow[j] = wd + ((long)e * H + (wv[j] ? c0 + j * 16 + r16 : 0)) * F;
+  }
+  f32x4 acc[2][NJ];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  u32x4 a[2], w[NJ], an[2], wn[NJ];
+  auto load = [&](u32x4 (&fa)[2], u32x4 (&fw)[NJ], int k0) {
+    const int k = k0 + kq * VEC;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[i] = load_frag<T>(arow[i], k, F, av[i], vec_ok);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) fw[j] = load_frag<T>(wrow[j], k, F, wv[j], vec_ok);
+  };
+  load(a, w, 0);
+  for (int k0 = 0; k0 < F; k0 += KS) {
+    if (k0 + KS < F) load(an, wn, k0 + KS);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) acc[i][j] = mma_frag(T{}, a[i], w[j], acc[i][j]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a[i] = an[i];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) w[j] = wn[j];
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int col = c0 + j * 16 + r16;
+      if (col >= H) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) y[(long)(tile * kMoeTile + i * 16 + kq * 4 + r) * H + col] = acc[i][j][r];
+    }
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
@@ -178,33 +252,46 @@ extern "C" void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int
   hipLaunchKernelGGL(dlia::moe_plan_kernel, dim3(1), dim3(1024), 0, stream, tiles, row_tok, pair_row, sel, pairs, top, E, max_rows);
 }
 
+// Steps with few rows (decoding) take narrow column blocks: more workgroups stream the experts' weights at once.
+template <typename T, typename OT, int NJ>
+static void launch_moe_up(void* act, const void* x, const void* wg, const void* wu, const int* tiles, const int* row_tok, int max_tiles,
+                          int F, int K, long ldx, long lda, float limit, int ok, hipStream_t stream) {
+  const dim3 grid((F + 64 * NJ - 1) / (64 * NJ), max_tiles);
+  hipLaunchKernelGGL((dlia::moe_up_kernel<T, OT, NJ>), grid, dim3(256), 0, stream, (OT*)act, (const T*)x, (const T*)wg, (const T*)wu,
+                     tiles, row_tok, F, K, ldx, lda, limit, ok);
+}
+template <typename T, int NJ>
+static void launch_moe_down(float* y, const void* act, const void* wd, const int* tiles, const int* row_tok, int max_tiles, int H, int F,
+                            long lda, int ok, hipStream_t stream) {
+  const dim3 grid((H + 64 * NJ - 1) / (64 * NJ), max_tiles);
+  hipLaunchKernelGGL((dlia::moe_down_kernel<T, NJ>), grid, dim3(256), 0, stream, y, (const T*)act, (const T*)wd, tiles, row_tok, H, F, lda, ok);
+}
+
 extern "C" void dlia_moe_up(void* act, const void* x, const void* wg, const void* wu, int f32, const int* tiles, const int* row_tok,
-                            int max_tiles, int F, int K, long ldx, long lda, float limit, hipStream_t stream) {
+                            int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, hipStream_t stream) {
   if (max_tiles <= 0) return;
-  const dim3 grid((F + 63) / 64, max_tiles);
+  const int vec = f32 ? 4 : 8;
+  const int ok = K % vec == 0 && ldx % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)wg % 16 == 0 && (uintptr_t)wu % 16 == 0;
   if (f32) {
-    const int ok = K % 4 == 0 && ldx % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)wg % 16 == 0 && (uintptr_t)wu % 16 == 0;
-    hipLaunchKernelGGL((dlia::moe_up_kernel<float, float>), grid, dim3(256), 0, stream, (float*)act, (const float*)x,
-                       (const float*)wg, (const float*)wu, tiles, row_tok, F, K, ldx, lda, limit, ok);
+    if (wide) launch_moe_up<float, float, 2>(act, x, wg, wu, tiles, row_tok, max_tiles, F, K, ldx, lda, limit, ok, stream);
+    else launch_moe_up<float, float, 1>(act, x, wg, wu, tiles, row_tok, max_tiles, F, K, ldx, lda, limit, ok, stream);
   } else {
-    const int ok = K % 8 == 0 && ldx % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)wg % 16 == 0 && (uintptr_t)wu % 16 == 0;
-    hipLaunchKernelGGL((dlia::moe_up_kernel<dlia::bf16, dlia::bf16>), grid, dim3(256), 0, stream, (dlia::bf16*)act,
-                       (const dlia::bf16*)x, (const dlia::bf16*)wg, (const dlia::bf16*)wu, tiles, row_tok, F, K, ldx, lda, limit, ok);
+    if (wide) launch_moe_up<dlia::bf16, dlia::bf16, 2>(act, x, wg, wu, tiles, row_tok, max_tiles, F, K, ldx, lda, limit, ok, stream);
+    else launch_moe_up<dlia::bf16, dlia::bf16, 1>(act, x, wg, wu, tiles, row_tok, max_tiles, F, K, ldx, lda, limit, ok, stream);
   }
 }
 
 extern "C" void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok,
-                              int max_tiles, int H, int F, long lda, hipStream_t stream) {
+                              int max_tiles, int wide, int H, int F, long lda, hipStream_t stream) {
   if (max_tiles <= 0) return;
-  const dim3 grid((H + 63) / 64, max_tiles);
+  const int vec = f32 ? 4 : 8;
+  const int ok = F % vec == 0 && lda % vec == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)wd % 16 == 0;
   if (f32) {
-    const int ok = F % 4 == 0 && lda % 4 == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)wd % 16 == 0;
-    hipLaunchKernelGGL(dlia::moe_down_kernel<float>, grid, dim3(256), 0, stream, y, (const float*)act, (const float*)wd, tiles,
-                       row_tok, H, F, lda, ok);
+    if (wide) launch_moe_down<float, 4>(y, act, wd, tiles, row_tok, max_tiles, H, F, lda, ok, stream);
+    else launch_moe_down<float, 1>(y, act, wd, tiles, row_tok, max_tiles, H, F, lda, ok, stream);
   } else {
-    const int ok = F % 8 == 0 && lda % 8 == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)wd % 16 == 0;
-    hipLaunchKernelGGL(dlia::moe_down_kernel<dlia::bf16>, grid, dim3(256), 0, stream, y, (const dlia::bf16*)act,
-                       (const dlia::bf16*)wd, tiles, row_tok, H, F, lda, ok);
+    if (wide) launch_moe_down<dlia::bf16, 4>(y, act, wd, tiles, row_tok, max_tiles, H, F, lda, ok, stream);
+    else launch_moe_down<dlia::bf16, 1>(y, act, wd, tiles, row_tok, max_tiles, H, F, lda, ok, stream);
   }
 }
 

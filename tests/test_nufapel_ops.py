@@ -295,10 +295,10 @@ def test_routed_ff_hip(T, W, E, top, ff, groups, keep, scale, limit, dt):
     x = _dev(h, at)
     logits = (_dev(h) @ _dev(t["x.router"]).T).contiguous()
     stack = lambda k: _dev(torch.stack([t[f"x.e{e}.{k}"] for e in range(E)]), at)
-    nt = (T * top + 15) // 16 + E
+    nt = (T * top + 31) // 32 + E
     i32 = lambda n: torch.zeros(n, dtype=torch.int32, device="cuda")
-    sel, wts, pair_row, tiles, row_tok = i32(T * top), torch.zeros(T * top, device="cuda"), i32(T * top), i32(1 + nt), i32(16 * nt)
-    eact, ey, out = torch.zeros(16 * nt, ff, device="cuda", dtype=at), torch.zeros(16 * nt, W, device="cuda"), torch.zeros(T, W, device="cuda")
+    sel, wts, pair_row, tiles, row_tok = i32(T * top), torch.zeros(T * top, device="cuda"), i32(T * top), i32(1 + nt), i32(32 * nt)
+    eact, ey, out = torch.zeros(32 * nt, ff, device="cuda", dtype=at), torch.zeros(32 * nt, W, device="cuda"), torch.zeros(T, W, device="cuda")
     for _ in range(2):                                   # (a second run over the same buffers: nothing is left over from the first)
         K.moe_route(sel, wts, logits, top, groups, keep, scale)
         K.moe_plan(tiles, row_tok, pair_row, sel, T * top, top, E)
