@@ -15,8 +15,9 @@
 // load a chunk's per-token vectors and evaluate the gates (a token per 16 lanes), then every lane walks the chunk's tokens
 // over its registers. A step is ragged: sequence b brings q_start[b+1] - q_start[b] tokens after ctx[b] earlier ones and
 // owns state slot slots[b]; ctx 0 starts from zeros (m from 0) whatever the slot held, so slots change hands without clearing.
-// The running maximum is kept once per column block (mstate [slots, H, kScanMaxBlocks]), so that no workgroup reads what
-// another one writes.
+// The running maximum is kept in kScanMaxBlocks copies per (slot, head): the workgroup of column block zb (of ZB) reads copy zb
+// and writes every copy whose index is zb modulo ZB, so that no workgroup reads what another one of the same launch writes,
+// and a later step that splits the columns into another number of blocks still finds every copy it reads up to date.
 #include <stdlib.h>
 #include "common.h"
 #include "launch.h"
@@ -33,7 +34,7 @@ struct ScanArgs {
   float* state; float* mstate;
   const float* b0; const float* b1;
   const int* q_start; const int* ctx; const int* slots;
-  int H, d, dv, NC, R, CB, CH, DP, state_rows;
+  int H, d, dv, NC, R, CB, CH, DP, state_rows, ZB;
   int col_q, col_k, col_v, col_a, col_i, col_f;
   float cap, qscale;
 };
@@ -161,12 +162,14 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
       if (row < d) S[(long)row * NC + j] = s[e];
     }
   }
-  if (RULE == 1 && tid == 0) mp[0] = m_run;
+  if (RULE == 1 && tid == 0)
+    for (int i = zb; i < kScanMaxBlocks; i += p.ZB) mp[i - zb] = m_run;
 }
 
 // The same walk for key sizes up to 128 with everything that sits on the chain from one token to the next made short. A
 // workgroup's four waves each sit alone on a SIMD, so nothing hides latency: the time per token IS the dependent chain. Here
-// a column's rows are spread over R <= 8 lanes known at compile time (16 rows each; in LDS every 16 rows are followed by 4 words
+// a column's rows are spread over R <= 16 lanes known at compile time (16 rows each, or 8 when a step has so few sequences
+// that narrower column blocks are what fills the chip; in LDS every lane's rows are followed by 4 words
 // of padding, so that the 16-byte reads of lanes with different rows fall into different banks: without it the reads of a wave
 // collide four ways and the LDS pipe, not the arithmetic, sets the time per token), the two sums over the rows run as four
 // independent chains and finish with data-parallel-primitive moves between neighbouring lanes (no LDS round trip), the NEXT
@@ -174,12 +177,12 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
 // normalised) after it. Rule 1's running maximum is a prefix scan over the chunk's tokens in the (max, +) algebra —
 // m -> max(a + m, b) composes as (a1 + a2, max(a2 + b1, b2)) — done by the first 16 lanes of every wave with shuffles, so it
 // costs no barrier and no serial loop; the per-token factors then travel by lane broadcast.
-constexpr int kFastRows = 16, kFastPad = 4;
+constexpr int kFastPad = 4;
 
-template <int RULE, int R>
+template <int RULE, int R, int kFastRows>
 __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int NV = RULE == 0 ? 5 : 2, CB = 256 / R, DP = (kFastRows + kFastPad) * R, CH = 16, VPL = CB / 16, EL = R;
+  constexpr int NV = RULE == 0 ? 5 : 2, CB = 256 / R, DP = (kFastRows + kFastPad) * R, CH = 16, VPL = CB / 16, EL = kFastRows * R / 16;
   auto at = [](int row) { return row + (row / kFastRows) * kFastPad; };      // a row's place in a padded vector
   const int b = blockIdx.x, h = blockIdx.y, zb = blockIdx.z;
   const int t0 = p.q_start[b], n = p.q_start[b + 1] - t0, c0 = p.ctx[b], slot = p.slots[b];
@@ -342,18 +345,23 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
     }
   }
   if constexpr (RULE == 1) {
-    if (tid == 0) mp[0] = m_run;
+    if (tid == 0)
+      for (int i = zb; i < kScanMaxBlocks; i += p.ZB) mp[i - zb] = m_run;
   }
 }
 
-template <int RULE>
+template <int RULE, int ROWS>
 static void launch_scan_fast(const ScanArgs& p, int R, dim3 grid, hipStream_t stream) {
   const int nv = RULE == 0 ? 5 : 2;
-  const size_t lds = (size_t)16 * (nv * (kFastRows + kFastPad) * R + 256 / R + 2) * sizeof(float);
-  if (R == 1) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 1>), grid, dim3(256), lds, stream, p);
-  else if (R == 2) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 2>), grid, dim3(256), lds, stream, p);
-  else if (R == 4) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 4>), grid, dim3(256), lds, stream, p);
-  else hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 8>), grid, dim3(256), lds, stream, p);
+  const size_t lds = (size_t)16 * (nv * (ROWS + kFastPad) * R + 256 / R + 2) * sizeof(float);
+  if constexpr (ROWS == 16) {
+    if (R == 1) { hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 1, 16>), grid, dim3(256), lds, stream, p); return; }
+  } else {
+    if (R == 16) { hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 16, 8>), grid, dim3(256), lds, stream, p); return; }
+  }
+  if (R == 2) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 2, ROWS>), grid, dim3(256), lds, stream, p);
+  else if (R == 4) hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 4, ROWS>), grid, dim3(256), lds, stream, p);
+  else hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 8, ROWS>), grid, dim3(256), lds, stream, p);
 }
 
 }  // namespace dlia
@@ -385,17 +393,23 @@ extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, lon
   p.CH = CH > 16 ? 16 : (CH < 1 ? 1 : CH);
   p.col_q = col_q; p.col_k = col_k; p.col_v = col_v; p.col_a = col_a; p.col_i = col_i; p.col_f = col_f; p.cap = cap; p.qscale = qscale;
   const int ZB = (p.NC + p.CB - 1) / p.CB;
-  if (ZB > dlia::kScanMaxBlocks) return 2;
+  if (ZB > dlia::kScanMaxBlocks / 2) return 2;
+  p.ZB = ZB;
   const size_t lds = (size_t)p.CH * per_token * sizeof(float);
   const dim3 grid(B, H, ZB);
   static const bool fast_on = [] { const char* e = getenv("DLIA_SCAN_FAST"); return !(e && atoi(e) == 0); }();
   // (steps of few tokens per sequence — decoding — run many workgroups at once: there the kernel that needs a third of the
   // registers keeps more of them resident, and there is no chain of tokens to shorten)
-  if (d <= 8 * dlia::kFastRows && fast_on && max_q >= 8) {
-    int Rf = 1;
-    while (Rf * dlia::kFastRows < d) Rf <<= 1;
-    const dim3 gridf(B, H, (p.NC + 256 / Rf - 1) / (256 / Rf));
-    if (rule == 0) dlia::launch_scan_fast<0>(p, Rf, gridf, stream); else dlia::launch_scan_fast<1>(p, Rf, gridf, stream);
+  if (d <= 128 && fast_on && max_q >= 8) {
+    // few workgroups (one long prompt): 8 rows per lane, twice the column blocks, half the work per token and lane
+    const bool narrow = d > 8 && (long)B * H * ZB < 192;
+    const int rows = narrow ? 8 : 16;
+    int Rf = narrow ? 2 : 1;
+    while (Rf * rows < d) Rf <<= 1;
+    p.ZB = (p.NC + 256 / Rf - 1) / (256 / Rf);
+    const dim3 gridf(B, H, p.ZB);
+    if (narrow) { if (rule == 0) dlia::launch_scan_fast<0, 8>(p, Rf, gridf, stream); else dlia::launch_scan_fast<1, 8>(p, Rf, gridf, stream); }
+    else { if (rule == 0) dlia::launch_scan_fast<0, 16>(p, Rf, gridf, stream); else dlia::launch_scan_fast<1, 16>(p, Rf, gridf, stream); }
     return 0;
   }
   if (rule == 0)
