@@ -214,6 +214,33 @@ def test_greedy_generation_through_the_scheduler(models, backend, dtype, stack, 
             assert row[t] >= best - (1e-3 if dtype == "fp32" else 0.35) * max(1.0, abs(best)), (t, int(row.argmax()))
 
 
+@pytest.mark.parametrize("backend,dtype,model", [pytest.param("torch", "fp32", "tiny-nufapel-test", id="torch"),
+                                                 pytest.param("hip", "bf16", "tiny-nufapel-gpu-test", id="hip-bf16", marks=pytest.mark.gpu)])
+def test_builtin_stack_samples_reproducibly(backend, dtype, model):
+    """A built-in stack (random weights drawn by the package, no checkpoint) through the engine with temperature / top-k / top-p
+    sampling: the same seeds give the same tokens on a second pipeline, other seeds do not."""
+    from distributed_llm_inference_amd.config import EngineConfig
+    from distributed_llm_inference_amd.parallel.launcher import LocalPipeline
+    from distributed_llm_inference_amd.runtime.sampler import SamplingParams
+
+    def run(seeds):
+        ecfg = EngineConfig(model=model, dtype=dtype, pp_size=1, max_batch=4, num_micro_batches=1, max_seq_len=128, prefill_chunk=32,
+                            kv_blocks=16, device="cuda" if backend == "hip" else "cpu", backend=backend, seed=3)
+        pipe = LocalPipeline(ecfg)
+        try:
+            reqs = [pipe.engine.submit(list(range(3, 3 + n)), SamplingParams(temperature=3.0, top_k=40, top_p=0.95, max_new_tokens=12,
+                                                                              seed=s, stop_on_eos=False))
+                    for n, s in zip((4, 21, 40), seeds)]
+            return [r.wait(120).output for r in reqs]
+        finally:
+            pipe.close()
+
+    a, b, c = run((1, 2, 3)), run((1, 2, 3)), run((4, 5, 6))
+    assert all(len(o) == 12 for o in a)
+    assert a == b
+    assert a != c
+
+
 def _random_stack(seed: int):
     """A stack drawn at random: 2 to 5 layers of either kind in any order, any stretch repeated 1 to 3 times or none, head counts,
     groupings and sizes of all kinds, every feed-forward kind."""
