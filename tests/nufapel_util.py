@@ -125,7 +125,7 @@ STACKS = {
     # sizes the packed-weight GEMMs take in bf16 (inner sizes that are multiples of 128)
     "packed": make_config([gd_layer(2, 64, moe(8, 2, 128, 2, 1, 2.0), rank=16), par_layer(4, 2, 32, 32, 2, 64, 64, dense(256), rows=20, bias_max=300),
                            par_layer(8, 1, 16, 16, 1, 128, 128, moe(4, 2, 128, 2, 2, 1.0))], vocab=96, width=128, loop=(0, 2, 2)),
-    "mfma_heads": make_config([par_layer(4, 2, 64, 64, 2, 64, 64, dense(128), rows=14, bias_max=100), gd_layer(2, 64, None, rank=16),
+    "mfma_heads": make_config([par_layer(6, 2, 64, 64, 2, 64, 64, dense(128), rows=14, bias_max=100), gd_layer(2, 64, None, rank=16),
                                par_layer(8, 1, 128, 128, 1, 32, 48, moe(6, 2, 64, 3, 2, 1.5), scale=0.05, rows=24, bias_max=90)],
                               vocab=80, width=128, loop=(0, 3, 2)),
 }
