@@ -141,9 +141,10 @@ class LayerSpec:
 @dataclass(frozen=True)
 class MoeSpec:
     """A routed feed-forward: `experts` small gated feed-forwards of width `ff`, of which a token runs `top`.
-    Scores are the sigmoids of the router's logits. The experts form `groups` equal groups of neighbours; a
-    group's score is the sum of its two largest scores and only experts of the `keep` best groups can be
-    chosen. The chosen scores, divided by their sum and multiplied by `scale`, weigh the experts' outputs. An
+    Scores are the sigmoids of the router's logits. The experts are split into `groups` contiguous blocks of equal
+    size; a block is ranked by its best two scores added up, and the choice is made among the experts of the
+    `keep` best blocks. The outputs of the chosen experts are summed with weights score / (sum of the chosen
+    scores) * `scale`. An
     expert computes down(g sigmoid(1.702 g) (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), +-limit)."""
     experts: int
     top: int

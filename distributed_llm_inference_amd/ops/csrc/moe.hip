@@ -1,8 +1,8 @@
 // Routed feed-forward (mixture of experts) without a host round trip: routing, a plan that sorts the step's (token, choice)
 // pairs by expert into 32-row tiles, the experts' two GEMMs over those tiles, and the weighted sum per token.
 //
-//   moe_route    one thread per token. Scores are sigmoids of the fp32 router logits. Experts form `groups` equal groups of
-//                neighbours; a group's score is the sum of its two largest scores; the `keep` best groups stay; the `top`
+//   moe_route    one thread per token. Scores are sigmoids of the fp32 router logits. Experts are split into `groups` contiguous blocks of
+//                equal size; a block is ranked by its best two scores added up; the `keep` best blocks stay; the `top`
 //                best experts of those are chosen (equal scores: the lower index), weighted score / (sum + 1e-20) * scale.
 //   moe_plan     one workgroup. Counts the pairs per expert, lays the experts' row ranges out one after the other, each
 //                padded to whole 32-row tiles, and writes for every padded row its token (or -1), for every pair its row,
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ sel, fl
     int best = -1; float bs = -1.f;
     for (int g = 0; g < groups; ++g) {
       if (gmask[g >> 6] >> (g & 63) & 1ull) continue;
-      float a = -1.f, b = -1.f;                       // the two largest scores of the group
+      float a = -1.f, b = -1.f;                       // the block's best two scores
       for (int e = g * per; e < (g + 1) * per; ++e) {
         const float s = score(e);
         if (s > a) { b = a; a = s; } else if (s > b) b = s;

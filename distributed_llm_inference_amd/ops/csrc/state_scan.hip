@@ -1,7 +1,7 @@
 // Linear recurrences over a per-sequence matrix state, token by token, everything in fp32. One kernel, two rules:
 //
 //   rule 0, generalised delta rule, state S [d, d] per head:
-//       u = k / sqrt(sum k^2 + 1e-6);  S <- diag(w) S - (a u) (u^T S) + k v^T  (both terms read the old S);  o = S^T r
+//       u = k / sqrt(sum k^2 + 1e-6);  S <- diag(w) S - (a u) (u^T S) + k v^T  (S on the right is the state before the token);  o = S^T r
 //       w = exp(-exp(-1/2) sigmoid(wz + w0)),  a = sigmoid(za + ba)   (a decay and a removal rate per key channel)
 //   rule 1, matrix memory with exponential gates, state S [d, dv], normaliser n [d], running maximum m per head:
 //       i = cap tanh((zi + bi) / cap),  f = logsigmoid(cap tanh((zf + bf) / cap)),  m' = max(f + m, i)

@@ -131,8 +131,8 @@ def distance_bias_table(rel: torch.Tensor, far: int, distances: int) -> torch.Te
 
 
 def general_delta_rule(r, k, v, w, a, S, eps: float = 1e-6):
-    """Token by token, per head: u = k / sqrt(sum k^2 + eps); S <- diag(w) S - (a u) (u^T S) + k v^T (both terms read
-    the old state); o = S^T r. r, k, v, w, a [T, H, d], S [H, d, d] fp32. Returns (o [T, H, d], S)."""
+    """Token by token, per head: u = k / sqrt(sum k^2 + eps); S <- diag(w) S - (a u) (u^T S) + k v^T (decay and removal
+    both act on S as it was before the token); o = S^T r. r, k, v, w, a [T, H, d], S [H, d, d] fp32. Returns (o [T, H, d], S)."""
     rf, kf, vf, wf, af, S = r.float(), k.float(), v.float(), w.float(), a.float(), S.float().clone()
     u = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + eps)
     out = torch.empty_like(vf)
@@ -163,9 +163,9 @@ def matrix_memory(q, k, v, log_i, log_f, S, n, m):
 
 def moe_route(scores: torch.Tensor, top: int, groups: int, keep: int, scale: float):
     """scores [T, E] fp32 (sigmoids of the router's logits) -> (experts [T, top] int64, weights [T, top] fp32). Experts
-    form `groups` equal groups of neighbours; a group's score is the sum of its two largest scores, only experts of the
-    `keep` best groups can be chosen; the `top` largest of them are, weighted by score / (sum + 1e-20) * scale. Equal
-    scores go to the lower index."""
+    are split into `groups` contiguous blocks of equal size; a block is ranked by its best two scores added up; experts
+    outside the `keep` best blocks are out of the running; of the rest the `top` highest are taken, each weighted by
+    score / (sum of the taken scores + 1e-20) * scale. Equal scores go to the lower index."""
     T, E = scores.shape
     per = E // groups
     sf = scores.float()

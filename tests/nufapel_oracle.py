@@ -62,7 +62,7 @@ def biased_sink_attention(h, t, m, pre):
 
 
 def matrix_memory(h, t, m, pre, eps):
-    """A matrix memory with exponential gates kept in range by a running maximum mx (which starts at 0):
+    """A matrix memory with exponential gates stabilised by a running maximum mx whose initial value is 0, not -inf:
     mx_t = max(f + mx_(t-1), i); S_t = exp(f + mx_(t-1) - mx_t) S_(t-1) + exp(i - mx_t) k v^T, n_t the same with k alone;
     o_t = S_t^T q / (max(|n_t . q|, exp(-mx_t)) + 1e-6)."""
     T = h.shape[0]
