@@ -516,7 +516,7 @@ class HybridGpuStage(GpuStage):
                 K.unary_act(low, z[:, 5 * n:5 * n + R], 1)
                 self._mm(wk, wz, low, p, "w_w2")
                 K.state_scan(0, o, z, wz[:, :n], self.rec[ri][0], None, p["b_a"], p["w0"], q_start, ctx, slots, ls.heads, d, d,
-                             0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0, max_q)
+                             0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0, max_q, self.wmode == "bf16")
                 K.headnorm_gate(mixed, o, z[:, 3 * n:4 * n], p["o_norm_w"], ls.heads, d, 0, eps)
                 self._mm(wk, ya, mixed, p, "w_o")
                 g0, wa, wb = 5 * n + R, None, None
@@ -549,7 +549,7 @@ class HybridGpuStage(GpuStage):
                                        p["temp"], p["bias"], p["sink"], gate)
                 self._mm(wk, ya, mixed, p, "w_o")
                 K.state_scan(1, o, z, None, self.rec[ri][0], self.rec[ri][1], p["b_if"], None, q_start, ctx, slots, b.heads, b.dim, b.vdim,
-                             c_q, c_k, c_v, 0, c_i, c_i + b.heads, b.gate_cap, b.scale, max_q)
+                             c_q, c_k, c_v, 0, c_i, c_i + b.heads, b.gate_cap, b.scale, max_q, self.wmode == "bf16")
                 K.headnorm_gate(mixed2, o, z[:, c_rg:c_rg + bv], p["o_norm_w"], b.heads, b.vdim, 2, eps)
                 yb = view(wk.yb, self._cols(p, "w_o"))
                 self._mm(wk, yb, mixed2, p, "w_o_r")

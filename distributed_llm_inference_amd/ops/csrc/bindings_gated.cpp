@@ -167,7 +167,7 @@ int64_t state_scan_blocks(int64_t d, int64_t ncols) { return dlia_state_scan_blo
 void state_scan(int64_t rule, Tensor o, const Tensor& z, OptTensor wz, Tensor state, const std::optional<Tensor>& mstate,
                 const Tensor& b0, OptTensor b1, const Tensor& q_start, const Tensor& ctx, const Tensor& slots, int64_t H, int64_t d,
                 int64_t dv, int64_t col_q, int64_t col_k, int64_t col_v, int64_t col_a, int64_t col_i, int64_t col_f, double cap,
-                double qscale, int64_t max_q) {
+                double qscale, int64_t max_q, bool quick) {
   DLIA_ON_DEVICE_OF(o);
   check_fmat(o, "o"); check_fmat(z, "z"); check_f32(state, "state"); check_f32(b0, "b0");
   check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots");
@@ -198,7 +198,7 @@ void state_scan(int64_t rule, Tensor o, const Tensor& z, OptTensor wz, Tensor st
                                  state.data_ptr<float>(), const_cast<float*>(mp), b0.data_ptr<float>(),
                                  b1.has_value() ? b1->data_ptr<float>() : nullptr, q_start.data_ptr<int>(), ctx.data_ptr<int>(),
                                  slots.data_ptr<int>(), (int)B, (int)H, (int)d, (int)dv, (int)state.size(0), (int)col_q, (int)col_k,
-                                 (int)col_v, (int)col_a, (int)col_i, (int)col_f, (float)cap, (float)qscale, (int)max_q, cur_stream());
+                                 (int)col_v, (int)col_a, (int)col_i, (int)col_f, (float)cap, (float)qscale, (int)max_q, quick ? 1 : 0, cur_stream());
   DLIA_CHECK(rc == 0, "state_scan: key size ", d, " / value size ", dv, " beyond what the kernel splits (1024 rows, 128 column blocks)");
 }
 
@@ -266,7 +266,7 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("softcap(Tensor(a!) logits, int vocab, float cap) -> ()");
   m.def("biased_attention(Tensor(a!) out, Tensor qkv, Tensor kcache, Tensor vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int G, int d, int dv, float scale, Tensor? temp, Tensor? bias, Tensor? sink, Tensor? gate) -> ()");
   m.def("state_scan_blocks(int d, int ncols) -> int");
-  m.def("state_scan(int rule, Tensor(a!) o, Tensor z, Tensor? wz, Tensor(b!) state, Tensor(c!)? mstate, Tensor b0, Tensor? b1, Tensor q_start, Tensor ctx, Tensor slots, int H, int d, int dv, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap, float qscale, int max_q) -> ()");
+  m.def("state_scan(int rule, Tensor(a!) o, Tensor z, Tensor? wz, Tensor(b!) state, Tensor(c!)? mstate, Tensor b0, Tensor? b1, Tensor q_start, Tensor ctx, Tensor slots, int H, int d, int dv, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap, float qscale, int max_q, bool quick) -> ()");
   m.def("moe_route(Tensor(a!) sel, Tensor(b!) wts, Tensor logits, int top, int groups, int keep, float scale) -> ()");
   m.def("moe_plan(Tensor(a!) tiles, Tensor(b!) row_tok, Tensor(c!) pair_row, Tensor sel, int pairs, int top, int E) -> ()");
   m.def("moe_up(Tensor(a!) act, Tensor x, Tensor wg, Tensor wu, Tensor tiles, Tensor row_tok, int max_tiles, float limit) -> ()");

@@ -159,7 +159,7 @@ int dlia_state_scan_blocks(int d, int ncols);
 int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, const float* wz, long ldw, float* state, float* mstate,
                     const float* b0, const float* b1, const int* q_start, const int* ctx, const int* slots, int B, int H, int d,
                     int dv, int state_rows, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap,
-                    float qscale, int max_q, hipStream_t stream);
+                    float qscale, int max_q, int quick, hipStream_t stream);
 
 // ---- moe.hip --------------------------------------------------------------------------------
 void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, int E, int top, int groups, int keep, float scale,

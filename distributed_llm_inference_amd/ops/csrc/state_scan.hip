@@ -37,10 +37,16 @@ struct ScanArgs {
   int H, d, dv, NC, R, CB, CH, DP, state_rows, ZB;
   int col_q, col_k, col_v, col_a, col_i, col_f;
   float cap, qscale;
+  int quick;      // gates through the hardware's exp2 / reciprocal (about 1 ulp) instead of the library functions
 };
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float logsigmoidf_(float x) { return x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x)); }
+// the same gates on the hardware's transcendental instructions: still fp32, about 1 ulp each; the library versions are
+// a few dozen instructions per value, which is most of what a chunk costs besides walking its tokens
+__device__ __forceinline__ float q_exp(float x) { return __expf(x); }
+__device__ __forceinline__ float q_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+__device__ __forceinline__ float q_tanh(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f); }
 
 template <int RULE>
 __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs p) {
@@ -193,6 +199,7 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
   float* vec = lds;                                  // [CH][NV][DP]
   float* vals = vec + CH * NV * DP;                  // [CH][CB]
   float* sc = vals + CH * CB;                        // [CH][2]: rule 1: log i, log f
+  float* obuf = sc + CH * 2;                         // [CH][CB + 1]: the chunk's read-outs (and exp(-m')) until they are stored
   float* S = p.state + ((long)slot * p.H + h) * (long)d * NC;
   float s[kFastRows];
 #pragma unroll
@@ -204,9 +211,16 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
   float m_run = 0.f;
   if constexpr (RULE == 1) m_run = c0 > 0 ? mp[0] : 0.f;
   const int tt = tid >> 4, sub = tid & 15, hd = h * d, lane = tid & 63;
-  float pa[EL], pb[EL], pc[RULE == 0 ? EL : 1], pd[RULE == 0 ? EL : 1], pv[VPL], pi = 0.f, pf = 0.f;
+  // Inputs on their way from memory: D chunks ahead, a register set each. All memory traffic of a chunk is issued at ONE
+  // point, between the two barriers: the read-outs of the chunk just walked (they wait in LDS) and the fetch of the chunk
+  // after the next. The vector-memory counter is a single in-order count, and a wait for fetched inputs behind a loop of
+  // conditional stores is a wait for everything; issued together and a whole walk ahead of the next wait, nothing stalls.
+  constexpr int D = 1;
+  struct Pre { float pa[EL], pb[EL], pc[RULE == 0 ? EL : 1], pd[RULE == 0 ? EL : 1], pv[VPL], pi, pf; };
+  Pre pre[D];
 
-  auto prefetch = [&](int ch0) {
+  auto prefetch = [&](Pre& r, int ch0) {
+    float (&pa)[EL] = r.pa; float (&pb)[EL] = r.pb; auto& pc = r.pc; auto& pd = r.pd; float (&pv)[VPL] = r.pv; float& pi = r.pi; float& pf = r.pf;
     if (tt >= min(CH, n - ch0)) return;
     const long t = t0 + ch0 + tt;
     const float* zr = p.z + t * p.ldz;
@@ -230,8 +244,10 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
       if (sub == 0) { pi = zr[p.col_i + h] + p.b0[h]; pf = zr[p.col_f + h] + p.b0[p.H + h]; }
     }
   };
-  auto commit = [&](int nt) {
+  auto commit = [&](const Pre& r, int nt) {
     if (tt >= nt) return;
+    const float (&pa)[EL] = r.pa; const float (&pb)[EL] = r.pb; const auto& pc = r.pc; const auto& pd = r.pd; const float (&pv)[VPL] = r.pv;
+    const float pi = r.pi, pf = r.pf;
     float* vt = vec + tt * NV * DP;
     if constexpr (RULE == 0) {
       float ksq = 0.f;
@@ -244,29 +260,42 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
         const bool ok = sub * EL + e < d;
         const float u = pa[e] * inv;
         float* v0 = vt + at(sub * EL + e);
-        v0[0] = ok ? expf(-0.6065306597126334f * sigmoidf_(pd[e])) : 0.f;
-        v0[DP] = ok ? sigmoidf_(pc[e]) * u : 0.f;
+        const float wv = p.quick ? q_exp(-0.6065306597126334f * q_sigmoid(pd[e])) : expf(-0.6065306597126334f * sigmoidf_(pd[e]));
+        const float av = p.quick ? q_sigmoid(pc[e]) : sigmoidf_(pc[e]);
+        v0[0] = ok ? wv : 0.f;
+        v0[DP] = ok ? av * u : 0.f;
         v0[2 * DP] = u; v0[3 * DP] = pa[e]; v0[4 * DP] = pb[e];
       }
     } else {
 #pragma unroll
       for (int e = 0; e < EL; ++e) { float* v0 = vt + at(sub * EL + e); v0[0] = pa[e]; v0[DP] = pb[e] * p.qscale; }
       if (sub == 0) {
-        sc[tt * 2] = p.cap * tanhf(pi / p.cap);
-        sc[tt * 2 + 1] = logsigmoidf_(p.cap * tanhf(pf / p.cap));
+        sc[tt * 2] = p.cap * (p.quick ? q_tanh(pi / p.cap) : tanhf(pi / p.cap));
+        sc[tt * 2 + 1] = logsigmoidf_(p.cap * (p.quick ? q_tanh(pf / p.cap) : tanhf(pf / p.cap)));
       }
     }
 #pragma unroll
     for (int e = 0; e < VPL; ++e) vals[tt * CB + sub * VPL + e] = pv[e];
   };
 
-  prefetch(0);
-  for (int ch0 = 0; ch0 < n; ch0 += CH) {
+  auto flush = [&](int ch0, int nt) {                // the read-outs of the chunk that starts at ch0, from LDS to memory
+    constexpr int HS = RULE == 0 ? 0 : 2;
+    for (int i = tid; i < nt * CB; i += 256) {
+      const int q = i / CB, cc = i % CB, jj = zb * CB + cc;
+      if (jj < NC) p.o[(long)(t0 + ch0 + q) * p.ldo + h * (p.dv + HS) + jj] = obuf[q * (CB + 1) + cc];
+    }
+    if constexpr (RULE == 1) {
+      if (tid < nt && zb * CB <= p.dv && p.dv < (zb + 1) * CB)
+        p.o[(long)(t0 + ch0 + tid) * p.ldo + h * (p.dv + 2) + p.dv + 1] = obuf[tid * (CB + 1) + CB];
+    }
+  };
+  auto chunk = [&](Pre& pr, int ch0) {
     const int nt = min(CH, n - ch0);
     __syncthreads();                                 // the previous chunk has been walked
-    commit(nt);
+    commit(pr, nt);
+    if (ch0 > 0) flush(ch0 - CH, CH);
+    if (ch0 + D * CH < n) prefetch(pr, ch0 + D * CH);      // in flight while this chunk is walked
     __syncthreads();
-    if (ch0 + CH < n) prefetch(ch0 + CH);            // in flight while this chunk is walked
     [[maybe_unused]] float keepv = 1.f, putv = 0.f, emv = 1.f;
     if constexpr (RULE == 1) {
       const bool live = lane < nt;
@@ -280,7 +309,8 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
       const float m_t = fmaxf(a + m_run, bb);
       float m_prev = __shfl_up(m_t, 1, 64);
       if ((lane & 15) == 0) m_prev = m_run;
-      keepv = expf(lf + m_prev - m_t); putv = expf(li - m_t); emv = expf(-m_t);
+      if (p.quick) { keepv = q_exp(lf + m_prev - m_t); putv = q_exp(li - m_t); emv = q_exp(-m_t); }
+      else { keepv = expf(lf + m_prev - m_t); putv = expf(li - m_t); emv = expf(-m_t); }
       m_run = __shfl(m_t, nt - 1, 64);
     }
     // two register sets: the vectors of token q + 1 are read from LDS while token q is applied
@@ -318,12 +348,10 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
         }
       }
       const float out = group_sum<R>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-      if (rg == 0 && col_ok) {
-        float* orow = p.o + (long)(t0 + ch0 + q) * p.ldo;
-        if constexpr (RULE == 0) orow[h * p.dv + j] = out;
-        else {
-          orow[h * (p.dv + 2) + j] = out;
-          if (j == p.dv) orow[h * (p.dv + 2) + p.dv + 1] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, emv), q));
+      if (rg == 0) {
+        obuf[q * (CB + 1) + c] = out;
+        if constexpr (RULE == 1) {
+          if (j == p.dv) obuf[q * (CB + 1) + CB] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, emv), q));
         }
       }
     };
@@ -336,7 +364,17 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
         apply(vb, xb, q + 1);
       }
     }
+  };
+#pragma unroll
+  for (int i = 0; i < D; ++i)
+    if (i * CH < n) prefetch(pre[i], i * CH);
+  for (int base = 0; base < n; base += D * CH) {
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (base + i * CH < n) chunk(pre[i], base + i * CH);
   }
+  __syncthreads();
+  flush((n - 1) / CH * CH, n - (n - 1) / CH * CH);
   if (col_ok) {
 #pragma unroll
     for (int e = 0; e < kFastRows; ++e) {
@@ -353,7 +391,7 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
 template <int RULE, int ROWS>
 static void launch_scan_fast(const ScanArgs& p, int R, dim3 grid, hipStream_t stream) {
   const int nv = RULE == 0 ? 5 : 2;
-  const size_t lds = (size_t)16 * (nv * (ROWS + kFastPad) * R + 256 / R + 2) * sizeof(float);
+  const size_t lds = (size_t)16 * (nv * (ROWS + kFastPad) * R + 2 * (256 / R) + 3) * sizeof(float);
   if constexpr (ROWS == 16) {
     if (R == 1) { hipLaunchKernelGGL((state_scan_fast_kernel<RULE, 1, 16>), grid, dim3(256), lds, stream, p); return; }
   } else {
@@ -378,7 +416,7 @@ extern "C" int dlia_state_scan_blocks(int d, int ncols) {
 extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, const float* wz, long ldw, float* state,
                                float* mstate, const float* b0, const float* b1, const int* q_start, const int* ctx,
                                const int* slots, int B, int H, int d, int dv, int state_rows, int col_q, int col_k, int col_v,
-                               int col_a, int col_i, int col_f, float cap, float qscale, int max_q, hipStream_t stream) {
+                               int col_a, int col_i, int col_f, float cap, float qscale, int max_q, int quick, hipStream_t stream) {
   if (B <= 0) return 0;
   dlia::ScanArgs p;
   p.o = o; p.ldo = ldo; p.z = z; p.ldz = ldz; p.wz = wz; p.ldw = ldw; p.state = state; p.mstate = mstate; p.b0 = b0; p.b1 = b1;
@@ -391,7 +429,7 @@ extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, lon
   const int per_token = nv * p.DP + p.CB + 4;
   int CH = 12000 / per_token;
   p.CH = CH > 16 ? 16 : (CH < 1 ? 1 : CH);
-  p.col_q = col_q; p.col_k = col_k; p.col_v = col_v; p.col_a = col_a; p.col_i = col_i; p.col_f = col_f; p.cap = cap; p.qscale = qscale;
+  p.col_q = col_q; p.col_k = col_k; p.col_v = col_v; p.col_a = col_a; p.col_i = col_i; p.col_f = col_f; p.cap = cap; p.qscale = qscale; p.quick = quick;
   const int ZB = (p.NC + p.CB - 1) / p.CB;
   if (ZB > dlia::kScanMaxBlocks / 2) return 2;
   p.ZB = ZB;

@@ -72,8 +72,9 @@ def test_general_delta_rule_torch(H, d):
 
 
 @gpu
+@pytest.mark.parametrize("quick", [False, True])
 @pytest.mark.parametrize("H,d", [(1, 8), (3, 24), (2, 64), (1, 80), (2, 128), (1, 272)])
-def test_general_delta_rule_hip(H, d):
+def test_general_delta_rule_hip(H, d, quick):
     """Ragged steps of three sequences over two calls: the state carries over in the slot, a sequence that starts (context 0)
     ignores what its slot held, chunks of the token loop end inside and at the end of a step."""
     from distributed_llm_inference_amd import ops
@@ -95,7 +96,7 @@ def test_general_delta_rule_hip(H, d):
         o = torch.zeros(z.shape[0], n, device="cuda")
         q0, c, s = _meta(ql, cx, sl)
         # (the three sequences share w0 / a.b here: one layer's vectors)
-        K.state_scan(0, o, z, wz, state, None, _dev(t0["x.a.b"]), _dev(t0["x.w0"]), q0, c, s, H, d, d, 0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0, max(ql))
+        K.state_scan(0, o, z, wz, state, None, _dev(t0["x.a.b"]), _dev(t0["x.w0"]), q0, c, s, H, d, d, 0, n, 2 * n, 4 * n, 0, 0, 1.0, 1.0, max(ql), quick)
         mixed = torch.zeros(z.shape[0], n, device="cuda")
         K.headnorm_gate(mixed, o, z[:, 3 * n:4 * n], _dev(t0["x.norm"]), H, d, 0, 1e-5)
         at = 0
@@ -137,8 +138,9 @@ def test_matrix_memory_torch(H, d, dv, cap):
 
 
 @gpu
+@pytest.mark.parametrize("quick", [False, True])
 @pytest.mark.parametrize("H,d,dv,cap", [(1, 8, 8, 15.0), (2, 24, 40, 3.0), (3, 16, 8, 30.0), (2, 64, 64, 15.0), (1, 128, 300, 10.0), (2, 40, 1, 8.0)])
-def test_matrix_memory_hip(H, d, dv, cap):
+def test_matrix_memory_hip(H, d, dv, cap, quick):
     from distributed_llm_inference_amd import ops
     K = ops.load()
     lens = [41, 2, 18]
@@ -157,7 +159,7 @@ def test_matrix_memory_hip(H, d, dv, cap):
         o = torch.zeros(z.shape[0], H * (dv + 2), device="cuda")
         q0, c, s = _meta(ql, cx, sl)
         K.state_scan(1, o, z, None, state, mstate, _dev(torch.cat([t0["x.i.b"], t0["x.f.b"]])), None, q0, c, s, H, d, dv,
-                     int(cq), int(ck), int(cv), 0, int(ci), int(cf), cap, d ** -0.5, max(ql))
+                     int(cq), int(ck), int(cv), 0, int(ci), int(cf), cap, d ** -0.5, max(ql), quick)
         mixed = torch.zeros(z.shape[0], H * dv, device="cuda")
         K.headnorm_gate(mixed, o, z[:, int(cg):int(cg) + H * dv], _dev(t0["x.norm"]), H, dv, 2, 1e-5)
         at = 0
