@@ -299,3 +299,30 @@ def test_random_stacks(tmp_path, seed, backend, dtype):
     else:   # (a random stack can put a position where bf16 rounding is magnified past any fixed bound: the schedule check stays)
         e = float(np.quantile(pos_errs(got, alone(path, backend, dtype, toks).astype(np.float64)), 0.9))
         assert e < 0.1, f"seed {seed}: differs from the whole prompt run alone by {e:.3g}"
+
+
+def test_trace_run_executable(models, tmp_path):
+    """The executable on a Nufapel checkpoint: the model class is chosen by config.json, steps arrive as JSON lines, logits
+    leave as little-endian fp32 files. (CPU: torch executor.)"""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg, W, path = models["no_loop"]
+    a, b = random_tokens(cfg, 40, 71), random_tokens(cfg, 9, 72)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:33], "want": [0, 32]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:2], "want": []}, {"id": "a", "tokens": a[33:34], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[34:], "want": [5]}, {"id": "b", "tokens": b[2:], "want": [6]}], "end": ["a", "b"]}]
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "trace_run")
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, exe, "--model", path, "--dtype", "float32", "--out", str(out), "--max-tokens", "128",
+                        "--backend", "torch", "--device", "cpu"], input="".join(json.dumps(s) + "\n" for s in steps),
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done ")] == ["done 0", "done 1", "done 2"]
+    ra, rb = oracle_logits(cfg, W, a), oracle_logits(cfg, W, b)
+    V = cfg["vocab"]
+    got = {n: np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, V) for n in (0, 1, 2)}
+    check(got[0], ra[[0, 32]], "fp32")
+    check(got[1], ra[[33]], "fp32")
+    check(got[2], np.stack([ra[39], rb[8]]), "fp32")
