@@ -469,7 +469,9 @@ class HybridGpuStage(GpuStage):
                 z2 = max(z2, self._cols(p, "w_ff"))
                 if ls.moe is not None:
                     e = ls.moe
-                    pairs, tiles, ef = max(pairs, rows * e.top), max(tiles, (rows * e.top + 31) // 32 + e.experts), max(ef, e.ff)
+                    # (rows of the experts' sorted copies: whole tiles of 32 rows, or of 128 for steps with many rows)
+                    pairs, ef = max(pairs, rows * e.top), max(ef, e.ff)
+                    tiles = max(tiles, (rows * e.top + 31) // 32 + e.experts, 4 * ((rows * e.top + 127) // 128 + e.experts))
                 else:
                     ac, yc = max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
         ws_floats = self._ws_floats
@@ -569,12 +571,15 @@ class HybridGpuStage(GpuStage):
                     g0 = ls.ff
                 else:
                     e = ls.moe
-                    nt = (T * e.top + 31) // 32 + e.experts          # row tiles of 32: at most this many hold a row
-                    eact, ey, ya = wk.eact[:32 * nt * e.ff].view(32 * nt, e.ff), wk.ey[:32 * nt * H].view(32 * nt, H), view(wk.ya, H)
+                    # row tiles: 128 rows through the LDS-tiled kernel when the step has many rows (bf16, inner sizes in whole
+                    # k-steps), else 32 rows through the register-tiled kernels; at most nt tiles hold a row
+                    tr = 128 if (self.wmode == "bf16" and T * e.top >= 1024 and H % 32 == 0 and e.ff % 32 == 0) else 32
+                    nt = (T * e.top + tr - 1) // tr + e.experts
+                    eact, ey, ya = wk.eact[:tr * nt * e.ff].view(tr * nt, e.ff), wk.ey[:tr * nt * H].view(tr * nt, H), view(wk.ya, H)
                     K.moe_route(wk.sel, wk.wts, z2[:, :e.experts], e.top, e.groups, e.keep, e.scale)
-                    K.moe_plan(wk.tiles, wk.row_tok, wk.pair_row, wk.sel, T * e.top, e.top, e.experts)
-                    K.moe_up(eact, xn, p["w_gate_e"], p["w_up_e"], wk.tiles, wk.row_tok, nt, e.limit)
-                    K.moe_down(ey, eact, p["w_down_e"], wk.tiles, wk.row_tok, nt)
+                    K.moe_plan(wk.tiles, wk.row_tok, wk.pair_row, wk.sel, T * e.top, e.top, e.experts, tr)
+                    K.moe_up(eact, xn, p["w_gate_e"], p["w_up_e"], wk.tiles, wk.row_tok, nt, e.limit, tr)
+                    K.moe_down(ey, eact, p["w_down_e"], wk.tiles, wk.row_tok, nt, tr)
                     K.moe_combine(ya, ey, wk.pair_row, wk.wts, e.top)
                     g0 = e.experts
                 step, nw, nb, na = opening(ri + 1)

@@ -213,38 +213,48 @@ void moe_route(Tensor sel, Tensor wts, const Tensor& logits, int64_t top, int64_
                  (int)groups, (int)keep, (float)scale, cur_stream());
 }
 
-void moe_plan(Tensor tiles, Tensor row_tok, Tensor pair_row, const Tensor& sel, int64_t pairs, int64_t top, int64_t E) {
+void moe_plan(Tensor tiles, Tensor row_tok, Tensor pair_row, const Tensor& sel, int64_t pairs, int64_t top, int64_t E, int64_t tile_rows) {
   DLIA_ON_DEVICE_OF(tiles);
   check_i32(tiles, "tiles"); check_i32(row_tok, "row_tok"); check_i32(pair_row, "pair_row"); check_i32(sel, "sel");
-  const int64_t max_tiles = (pairs + 31) / 32 + E;
+  DLIA_CHECK(tile_rows == 32 || tile_rows == 128, "moe: row tiles of 32 or 128");
+  const int64_t max_tiles = (pairs + tile_rows - 1) / tile_rows + E;
   DLIA_CHECK(E >= 1 && E <= 256 && top >= 1 && pairs >= 0 && sel.numel() >= pairs && pair_row.numel() >= pairs, "moe_plan: pairs");
-  DLIA_CHECK(tiles.numel() >= 1 + max_tiles && row_tok.numel() >= 32 * max_tiles, "moe_plan: room for pairs / 32 + E tiles of 32 rows");
+  DLIA_CHECK(tiles.numel() >= 1 + max_tiles && row_tok.numel() >= tile_rows * max_tiles, "moe_plan: room for pairs / tile_rows + E tiles");
   dlia_moe_plan(tiles.data_ptr<int>(), row_tok.data_ptr<int>(), pair_row.data_ptr<int>(), sel.data_ptr<int>(), (int)pairs, (int)top, (int)E,
-                (int)(32 * max_tiles), cur_stream());
+                (int)(tile_rows * max_tiles), (int)tile_rows, cur_stream());
+}
+
+static void check_big(int64_t tile_rows, const Tensor& a, int64_t K, const Tensor& w) {
+  DLIA_CHECK(tile_rows == 32 || tile_rows == 128, "moe: row tiles of 32 or 128");
+  if (tile_rows == 128)
+    DLIA_CHECK(a.scalar_type() == at::kBFloat16 && K % 32 == 0 && a.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(a.data_ptr()) % 16 == 0 &&
+               reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0, "moe: 128-row tiles need bf16, K a multiple of 32 and 16-byte aligned rows");
 }
 
 void moe_up(Tensor act, const Tensor& x, const Tensor& wg, const Tensor& wu, const Tensor& tiles, const Tensor& row_tok, int64_t max_tiles,
-            double limit) {
+            double limit, int64_t tile_rows) {
   DLIA_ON_DEVICE_OF(act);
   check_act(act, "act"); check_mat(act, "act"); check_act(x, "x"); check_mat(x, "x"); check_act(wg, "wg"); check_act(wu, "wu");
   check_i32(tiles, "tiles"); check_i32(row_tok, "row_tok");
   DLIA_CHECK(wg.dim() == 3 && wg.is_contiguous() && wu.is_contiguous() && wu.sizes() == wg.sizes() && wg.size(2) == x.size(1) &&
              x.scalar_type() == wg.scalar_type() && wu.scalar_type() == wg.scalar_type() && act.scalar_type() == x.scalar_type(),
              "moe_up: x [T, K], wg / wu [E, F, K], one type");
-  DLIA_CHECK(act.size(1) == wg.size(1) && act.size(0) >= 32 * max_tiles && row_tok.numel() >= 32 * max_tiles && tiles.numel() >= 1 + max_tiles,
-             "moe_up: act [32 max_tiles, F]");
+  check_big(tile_rows, x, x.size(1), wg);
+  DLIA_CHECK(act.size(1) == wg.size(1) && act.size(0) >= tile_rows * max_tiles && row_tok.numel() >= tile_rows * max_tiles && tiles.numel() >= 1 + max_tiles,
+             "moe_up: act [tile_rows max_tiles, F]");
   dlia_moe_up(act.data_ptr(), x.data_ptr(), wg.data_ptr(), wu.data_ptr(), is_f32(x), tiles.data_ptr<int>(), row_tok.data_ptr<int>(),
-              (int)max_tiles, x.size(0) > 256 ? 1 : 0, (int)wg.size(1), (int)wg.size(2), x.stride(0), act.stride(0), (float)limit, cur_stream());
+              (int)max_tiles, x.size(0) > 256 ? 1 : 0, (int)wg.size(1), (int)wg.size(2), x.stride(0), act.stride(0), (float)limit, (int)tile_rows, cur_stream());
 }
 
-void moe_down(Tensor y, const Tensor& act, const Tensor& wd, const Tensor& tiles, const Tensor& row_tok, int64_t max_tiles) {
+void moe_down(Tensor y, const Tensor& act, const Tensor& wd, const Tensor& tiles, const Tensor& row_tok, int64_t max_tiles, int64_t tile_rows) {
   DLIA_ON_DEVICE_OF(y);
   check_f32(y, "y"); check_act(act, "act"); check_mat(act, "act"); check_act(wd, "wd"); check_i32(tiles, "tiles"); check_i32(row_tok, "row_tok");
   DLIA_CHECK(wd.dim() == 3 && wd.is_contiguous() && wd.size(2) == act.size(1) && wd.scalar_type() == act.scalar_type(), "moe_down: wd [E, H, F]");
-  DLIA_CHECK(y.dim() == 2 && y.size(1) == wd.size(1) && y.size(0) >= 32 * max_tiles && act.size(0) >= 32 * max_tiles &&
-             row_tok.numel() >= 32 * max_tiles && tiles.numel() >= 1 + max_tiles, "moe_down: y [32 max_tiles, H]");
+  check_big(tile_rows, act, act.size(1), wd);
+  DLIA_CHECK(y.dim() == 2 && y.size(1) == wd.size(1) && y.size(0) >= tile_rows * max_tiles && act.size(0) >= tile_rows * max_tiles &&
+             row_tok.numel() >= tile_rows * max_tiles && tiles.numel() >= 1 + max_tiles, "moe_down: y [tile_rows max_tiles, H]");
   dlia_moe_down(y.data_ptr<float>(), act.data_ptr(), wd.data_ptr(), is_f32(act), tiles.data_ptr<int>(), row_tok.data_ptr<int>(),
-                (int)max_tiles, max_tiles > 64 ? 1 : 0, (int)wd.size(1), (int)wd.size(2), act.stride(0), cur_stream());
+                (int)max_tiles, max_tiles > 64 ? 1 : 0, (int)wd.size(1), (int)wd.size(2), act.stride(0), (int)tile_rows, cur_stream());
 }
 
 void moe_combine(Tensor out, const Tensor& y, const Tensor& pair_row, const Tensor& wts, int64_t top) {
@@ -268,9 +278,9 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("state_scan_blocks(int d, int ncols) -> int");
   m.def("state_scan(int rule, Tensor(a!) o, Tensor z, Tensor? wz, Tensor(b!) state, Tensor(c!)? mstate, Tensor b0, Tensor? b1, Tensor q_start, Tensor ctx, Tensor slots, int H, int d, int dv, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap, float qscale, int max_q, bool quick) -> ()");
   m.def("moe_route(Tensor(a!) sel, Tensor(b!) wts, Tensor logits, int top, int groups, int keep, float scale) -> ()");
-  m.def("moe_plan(Tensor(a!) tiles, Tensor(b!) row_tok, Tensor(c!) pair_row, Tensor sel, int pairs, int top, int E) -> ()");
-  m.def("moe_up(Tensor(a!) act, Tensor x, Tensor wg, Tensor wu, Tensor tiles, Tensor row_tok, int max_tiles, float limit) -> ()");
-  m.def("moe_down(Tensor(a!) y, Tensor act, Tensor wd, Tensor tiles, Tensor row_tok, int max_tiles) -> ()");
+  m.def("moe_plan(Tensor(a!) tiles, Tensor(b!) row_tok, Tensor(c!) pair_row, Tensor sel, int pairs, int top, int E, int tile_rows) -> ()");
+  m.def("moe_up(Tensor(a!) act, Tensor x, Tensor wg, Tensor wu, Tensor tiles, Tensor row_tok, int max_tiles, float limit, int tile_rows) -> ()");
+  m.def("moe_down(Tensor(a!) y, Tensor act, Tensor wd, Tensor tiles, Tensor row_tok, int max_tiles, int tile_rows) -> ()");
   m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor pair_row, Tensor wts, int top) -> ()");
 }
 

@@ -164,12 +164,13 @@ int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, cons
 // ---- moe.hip --------------------------------------------------------------------------------
 void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, int E, int top, int groups, int keep, float scale,
                     hipStream_t stream);
-void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows,
+void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows, int tile_rows,
                    hipStream_t stream);
+// tile_rows: 32 (register-tiled expert kernels, any type and shape) or 128 (LDS-tiled, bf16, K a multiple of 32, aligned rows)
 void dlia_moe_up(void* act, const void* x, const void* wg, const void* wu, int f32, const int* tiles, const int* row_tok,
-                 int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, hipStream_t stream);
+                 int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, int tile_rows, hipStream_t stream);
 void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok, int max_tiles, int wide,
-                   int H, int F, long lda, hipStream_t stream);
+                   int H, int F, long lda, int tile_rows, hipStream_t stream);
 // (wide: 128 / 256 output columns per workgroup, for steps with many rows; else 64)
 void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
                       hipStream_t stream);

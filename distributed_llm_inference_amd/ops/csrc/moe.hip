@@ -20,7 +20,8 @@
 namespace dlia {
 
 constexpr int kMoeMaxExperts = 256;
-constexpr int kMoeRows = 32;           // rows of a plan tile
+constexpr int kMoeRows = 32;           // rows of a plan tile (steps with few rows), kMoeBigRows for the LDS-tiled kernel
+constexpr int kMoeBigRows = 128;
 
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ sel, float* __restrict__ wts,
                                                        const float* __restrict__ logits, long ld, int T, int E, int top,
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ sel, fl
 // tiles: [0] number of tiles, [1 + i] expert of tile i. row_tok [max_rows], pair_row [T * top].
 __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles, int* __restrict__ row_tok,
                                                         int* __restrict__ pair_row, const int* __restrict__ sel, int pairs,
-                                                        int top, int E, int max_rows) {
+                                                        int top, int E, int max_rows, int tile_rows) {
   __shared__ int count[kMoeMaxExperts], start[kMoeMaxExperts], fill[kMoeMaxExperts];
   __shared__ int ntiles;
   for (int e = threadIdx.x; e < E; e += 1024) { count[e] = 0; fill[e] = 0; }
@@ -79,15 +80,15 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles,
     int at = 0, nt = 0;
     for (int e = 0; e < E; ++e) {
       start[e] = at;
-      const int n = (count[e] + kMoeRows - 1) / kMoeRows;
+      const int n = (count[e] + tile_rows - 1) / tile_rows;
       for (int i = 0; i < n; ++i) tiles[1 + nt + i] = e;
-      nt += n; at += n * kMoeRows;
+      nt += n; at += n * tile_rows;
     }
     tiles[0] = nt;
     ntiles = nt;
   }
   __syncthreads();
-  const int used = ntiles * kMoeRows;
+  const int used = ntiles * tile_rows;
   for (int i = threadIdx.x; i < max_rows; i += 1024) row_tok[i] = -1;
   __syncthreads();
   for (int i = threadIdx.x; i < pairs; i += 1024) {
@@ -227,6 +228,100 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ y, co
     }
 }
 
+// Steps with many rows (prompts): 128-row tiles, operands staged through LDS. A workgroup owns one row tile by 128 weight rows —
+// for the up projection 64 gate rows and the 64 up rows of the same columns, so the activation is formed in registers; for the
+// down projection 128 output columns — and walks K in steps of 32: every thread brings four 16-byte pieces of the next step
+// (two of the rows, gathered through the plan for the up projection; two of the weights) into registers while the current
+// step is multiplied, then parks them in the other half of a double buffer. Rows are 80 bytes apart in LDS, which spreads the
+// fragment reads of a 16-row tile over the banks. A wave multiplies 32 rows by all 128 weight rows: 10 fragment reads for 16
+// MFMAs. bf16, K a multiple of 32 with 16-byte aligned rows (the caller falls back to the register-tiled kernels otherwise).
+constexpr int kBigStride = 40;          // bf16 elements between rows in LDS (64 bytes of data + 16 of padding)
+
+template <bool UP>
+__global__ __launch_bounds__(256) void moe_big_kernel(bf16* __restrict__ act_out, float* __restrict__ y_out, const bf16* __restrict__ a,
+                                                      const bf16* __restrict__ w0, const bf16* __restrict__ w1,
+                                                      const int* __restrict__ tiles, const int* __restrict__ row_tok, int N, int K,
+                                                      long lda, long ldo, float limit) {
+  __shared__ __attribute__((aligned(16))) bf16 lds[2][256 * kBigStride];
+  const int tile = blockIdx.y;
+  if (tile >= tiles[0]) return;
+  const int e = tiles[1 + tile];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r16 = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * (UP ? 64 : 128);                  // first output column of the workgroup
+  // the four pieces this thread stages per k-step: pieces 2 tid, 2 tid + 1 of the 512 row pieces, and of the 512 weight pieces
+  const bf16* src[4]; bool ok[4]; int dst[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int c = tid * 2 + i, row = c >> 2, part = c & 3;
+    const int grow = tile * kMoeBigRows + row;
+    if constexpr (UP) { const int tok = row_tok[grow]; ok[i] = tok >= 0; src[i] = a + (long)(ok[i] ? tok : 0) * lda + part * 8; }
+    else { ok[i] = row_tok[grow] >= 0; src[i] = a + (long)grow * lda + part * 8; }
+    dst[i] = row * kBigStride + part * 8;
+    // weights: LDS rows 128 .. 255
+    int wr; const bf16* base;
+    if constexpr (UP) { wr = n0 + (row & 63); base = row < 64 ? w0 : w1; }
+    else { wr = n0 + row; base = w0; }
+    ok[2 + i] = wr < N;
+    src[2 + i] = base + ((long)e * N + (ok[2 + i] ? wr : 0)) * K + part * 8;
+    dst[2 + i] = (128 + row) * kBigStride + part * 8;
+  }
+  u32x4 st[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st[i] = ok[i] ? ld16(src[i] + k0) : u32x4{0u, 0u, 0u, 0u};
+  };
+  auto park = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&lds[buf][dst[i]]) = st[i];
+  };
+  f32x4 acc[2][8];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  park(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool more = k0 + 32 < K;
+    if (more) fetch(k0 + 32);
+    u32x4 fa[2], fw[8];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const u32x4*>(&lds[buf][(wave * 32 + i * 16 + r16) * kBigStride + kq * 8]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fw[j] = *reinterpret_cast<const u32x4*>(&lds[buf][(128 + j * 16 + r16) * kBigStride + kq * 8]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = mfma16(fa[i], fw[j], acc[i][j]);
+    if (more) park(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const long row = (long)tile * kMoeBigRows + wave * 32 + i * 16 + kq * 4 + r;
+      if constexpr (UP) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int col = n0 + j * 16 + r16;
+          if (col >= N) continue;
+          const float gv = fminf(acc[i][j][r], limit), uv = fminf(fmaxf(acc[i][j + 4][r], -limit), limit);
+          act_out[row * ldo + col] = (bf16)(gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int col = n0 + j * 16 + r16;
+          if (col < N) y_out[row * ldo + col] = acc[i][j][r];
+        }
+      }
+    }
+}
+
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
                                                           const int* __restrict__ pair_row, const float* __restrict__ wts,
                                                           int H, int top, long ldo) {
@@ -248,8 +343,9 @@ extern "C" void dlia_moe_route(int* sel, float* wts, const float* logits, long l
 }
 
 extern "C" void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows,
-                              hipStream_t stream) {
-  hipLaunchKernelGGL(dlia::moe_plan_kernel, dim3(1), dim3(1024), 0, stream, tiles, row_tok, pair_row, sel, pairs, top, E, max_rows);
+                              int tile_rows, hipStream_t stream) {
+  hipLaunchKernelGGL(dlia::moe_plan_kernel, dim3(1), dim3(1024), 0, stream, tiles, row_tok, pair_row, sel, pairs, top, E, max_rows,
+                     tile_rows);
 }
 
 // Steps with few rows (decoding) take narrow column blocks: more workgroups stream the experts' weights at once.
@@ -268,8 +364,13 @@ static void launch_moe_down(float* y, const void* act, const void* wd, const int
 }
 
 extern "C" void dlia_moe_up(void* act, const void* x, const void* wg, const void* wu, int f32, const int* tiles, const int* row_tok,
-                            int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, hipStream_t stream) {
+                            int max_tiles, int wide, int F, int K, long ldx, long lda, float limit, int tile_rows, hipStream_t stream) {
   if (max_tiles <= 0) return;
+  if (tile_rows == dlia::kMoeBigRows) {
+    hipLaunchKernelGGL(dlia::moe_big_kernel<true>, dim3((F + 63) / 64, max_tiles), dim3(256), 0, stream, (dlia::bf16*)act, (float*)nullptr,
+                       (const dlia::bf16*)x, (const dlia::bf16*)wg, (const dlia::bf16*)wu, tiles, row_tok, F, K, ldx, lda, limit);
+    return;
+  }
   const int vec = f32 ? 4 : 8;
   const int ok = K % vec == 0 && ldx % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)wg % 16 == 0 && (uintptr_t)wu % 16 == 0;
   if (f32) {
@@ -282,8 +383,13 @@ extern "C" void dlia_moe_up(void* act, const void* x, const void* wg, const void
 }
 
 extern "C" void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int* tiles, const int* row_tok,
-                              int max_tiles, int wide, int H, int F, long lda, hipStream_t stream) {
+                              int max_tiles, int wide, int H, int F, long lda, int tile_rows, hipStream_t stream) {
   if (max_tiles <= 0) return;
+  if (tile_rows == dlia::kMoeBigRows) {
+    hipLaunchKernelGGL(dlia::moe_big_kernel<false>, dim3((H + 127) / 128, max_tiles), dim3(256), 0, stream, (dlia::bf16*)nullptr, y,
+                       (const dlia::bf16*)act, (const dlia::bf16*)wd, (const dlia::bf16*)nullptr, tiles, row_tok, H, F, lda, (long)H, 0.f);
+    return;
+  }
   const int vec = f32 ? 4 : 8;
   const int ok = F % vec == 0 && lda % vec == 0 && (uintptr_t)act % 16 == 0 && (uintptr_t)wd % 16 == 0;
   if (f32) {

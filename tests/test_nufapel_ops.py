@@ -264,7 +264,7 @@ def _moe_case(T, W, E, top, ff, groups, keep, scale, limit, seed):
     return torch.randn(T, W, generator=g, dtype=F64), t, mlp
 
 
-MOE = [(50, 32, 6, 2, 24, 3, 2, 1.5, 1.0), (33, 40, 8, 3, 20, 4, 2, 0.7, 7.0), (20, 24, 5, 1, 8, 1, 1, 2.5, 0.5), (70, 64, 12, 5, 16, 12, 7, 1.0, 2.0),
+MOE = [(50, 32, 6, 2, 24, 3, 2, 1.5, 1.0), (600, 128, 8, 2, 64, 2, 1, 2.0, 1.5), (350, 96, 5, 3, 160, 1, 1, 1.0, 7.0), (33, 40, 8, 3, 20, 4, 2, 0.7, 7.0), (20, 24, 5, 1, 8, 1, 1, 2.5, 0.5), (70, 64, 12, 5, 16, 12, 7, 1.0, 2.0),
        (130, 128, 9, 3, 72, 3, 3, 3.0, 1.5)]
 
 
@@ -297,17 +297,19 @@ def test_routed_ff_hip(T, W, E, top, ff, groups, keep, scale, limit, dt):
     x = _dev(h, at)
     logits = (_dev(h) @ _dev(t["x.router"]).T).contiguous()
     stack = lambda k: _dev(torch.stack([t[f"x.e{e}.{k}"] for e in range(E)]), at)
-    nt = (T * top + 31) // 32 + E
     i32 = lambda n: torch.zeros(n, dtype=torch.int32, device="cuda")
-    sel, wts, pair_row, tiles, row_tok = i32(T * top), torch.zeros(T * top, device="cuda"), i32(T * top), i32(1 + nt), i32(32 * nt)
-    eact, ey, out = torch.zeros(32 * nt, ff, device="cuda", dtype=at), torch.zeros(32 * nt, W, device="cuda"), torch.zeros(T, W, device="cuda")
-    for _ in range(2):                                   # (a second run over the same buffers: nothing is left over from the first)
-        K.moe_route(sel, wts, logits, top, groups, keep, scale)
-        K.moe_plan(tiles, row_tok, pair_row, sel, T * top, top, E)
-        K.moe_up(eact, x, stack("gate"), stack("up"), tiles, row_tok, nt, limit)
-        K.moe_down(ey, eact, stack("down"), tiles, row_tok, nt)
-        K.moe_combine(out, ey, pair_row, wts, top)
-    _close(out, ref, 2e-4 if dt == "fp32" else 3e-2)
+    # row tiles of 32 (register-tiled kernels) and, in bf16 with inner sizes in whole k-steps, of 128 (LDS-tiled kernel)
+    for tr in ([32, 128] if dt == "bf16" and W % 32 == 0 and ff % 32 == 0 else [32]):
+        nt = (T * top + tr - 1) // tr + E
+        sel, wts, pair_row, tiles, row_tok = i32(T * top), torch.zeros(T * top, device="cuda"), i32(T * top), i32(1 + nt), i32(tr * nt)
+        eact, ey, out = torch.zeros(tr * nt, ff, device="cuda", dtype=at), torch.zeros(tr * nt, W, device="cuda"), torch.zeros(T, W, device="cuda")
+        for _ in range(2):                               # (a second run over the same buffers: nothing is left over from the first)
+            K.moe_route(sel, wts, logits, top, groups, keep, scale)
+            K.moe_plan(tiles, row_tok, pair_row, sel, T * top, top, E, tr)
+            K.moe_up(eact, x, stack("gate"), stack("up"), tiles, row_tok, nt, limit, tr)
+            K.moe_down(ey, eact, stack("down"), tiles, row_tok, nt, tr)
+            K.moe_combine(out, ey, pair_row, wts, top)
+        _close(out, ref, 2e-4 if dt == "fp32" else 3e-2, f"row tiles of {tr}")
 
 
 # ---- norms, gates, activations ---------------------------------------------------------------------------------------------
