@@ -126,6 +126,23 @@ def test_mixed_batches_and_reuse(models, stack, backend, dtype):
 
 
 @pytest.mark.parametrize("backend,dtype", BACKENDS)
+def test_long_prompt(tmp_path, backend, dtype):
+    """A prompt long enough that the routed feed-forward takes its many-row path (128-row expert tiles on the GPU in bf16), the
+    recurrences walk dozens of chunks and the attention spans twenty cache blocks; whole, and in two portions."""
+    cfg = dict(STACKS["packed"], max_positions=1024)
+    W = random_weights(cfg, seed=77)
+    path = save(str(tmp_path / "m"), cfg, W)
+    toks = random_tokens(cfg, 640, 9)
+    ref = oracle_logits(cfg, W, toks)
+    whole = alone(path, backend, dtype, toks)
+    check(whole, ref, dtype, "whole")
+    sess = session(path, backend, dtype, max_tokens=704)
+    got = replay(sess, {"a": toks}, [[("a", 300)], [("a", 340)]])["a"]
+    sess.close()
+    check(got, ref, dtype, "two portions", whole)
+
+
+@pytest.mark.parametrize("backend,dtype", BACKENDS)
 def test_slot_taken_over_starts_clean(models, backend, dtype):
     """One slot, one request after another: the second must not see the first one's states, running maxima or cache rows."""
     cfg, W, path = models["loop_mid"]
