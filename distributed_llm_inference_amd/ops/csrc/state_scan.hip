@@ -37,6 +37,7 @@ struct ScanArgs {
   int H, d, dv, NC, R, CB, CH, DP, state_rows, ZB;
   int col_q, col_k, col_v, col_a, col_i, col_f;
   float cap, qscale;
+  int vec4;       // every row and column offset of z / wz is a multiple of 4 floats and 16-byte aligned: 16-byte loads
   int quick;      // gates through the hardware's exp2 / reciprocal (about 1 ulp) instead of the library functions
 };
 
@@ -219,29 +220,56 @@ __global__ __launch_bounds__(256) void state_scan_fast_kernel(ScanArgs p) {
   struct Pre { float pa[EL], pb[EL], pc[RULE == 0 ? EL : 1], pd[RULE == 0 ? EL : 1], pv[VPL], pi, pf; };
   Pre pre[D];
 
-  auto prefetch = [&](Pre& r, int ch0) {
-    float (&pa)[EL] = r.pa; float (&pb)[EL] = r.pb; auto& pc = r.pc; auto& pd = r.pd; float (&pv)[VPL] = r.pv; float& pi = r.pi; float& pf = r.pf;
-    if (tt >= min(CH, n - ch0)) return;
-    const long t = t0 + ch0 + tt;
-    const float* zr = p.z + t * p.ldz;
+  // the biases of this lane's rows are the same for every token: read once
+  [[maybe_unused]] float ba[RULE == 0 ? EL : 1], bw[RULE == 0 ? EL : 1];
+  if constexpr (RULE == 0) {
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const int i = sub * EL + e;
-      const bool ok = i < d;
-      pa[e] = ok ? zr[p.col_k + hd + i] : 0.f;
-      pb[e] = ok ? zr[p.col_q + hd + i] : 0.f;
-      if constexpr (RULE == 0) {
-        pc[e] = ok ? zr[p.col_a + hd + i] + p.b0[hd + i] : 0.f;
-        pd[e] = ok ? p.wz[t * p.ldw + hd + i] + p.b1[hd + i] : 0.f;
+      ba[e] = i < d ? p.b0[hd + i] : 0.f;
+      bw[e] = i < d ? p.b1[hd + i] : 0.f;
+    }
+  }
+  // (a chunk's inputs are a few kilobytes per workgroup; fetched one float per lane and instruction they are dozens of
+  // poorly coalesced requests per wave and the fetch, not the walk, sets the time per chunk: 16 bytes per lane where the
+  // layout allows)
+  auto row4 = [&](float (&dst)[EL], const float* src) {
+    if constexpr (EL % 4 == 0) {
+      if (p.vec4) {
+#pragma unroll
+        for (int e = 0; e < EL; e += 4) {
+          const int i = sub * EL + e;
+          const f32x4 t = i < d ? *reinterpret_cast<const f32x4*>(src + i) : f32x4{0.f, 0.f, 0.f, 0.f};
+          dst[e] = t.x; dst[e + 1] = t.y; dst[e + 2] = t.z; dst[e + 3] = t.w;
+        }
+        return;
       }
+    }
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const int i = sub * EL + e;
+      dst[e] = i < d ? src[i] : 0.f;
+    }
+  };
+  auto prefetch = [&](Pre& r, int ch0) {
+    if (tt >= min(CH, n - ch0)) return;
+    const long t = t0 + ch0 + tt;
+    const float* zr = p.z + t * p.ldz;
+    row4(r.pa, zr + p.col_k + hd);
+    row4(r.pb, zr + p.col_q + hd);
+    if constexpr (RULE == 0) {
+      row4(r.pc, zr + p.col_a + hd);
+      row4(r.pd, p.wz + t * p.ldw + hd);
+#pragma unroll
+      for (int e = 0; e < EL; ++e) { r.pc[e] += ba[e]; r.pd[e] += bw[e]; }
     }
 #pragma unroll
     for (int e = 0; e < VPL; ++e) {
       const int jj = zb * CB + sub * VPL + e;
-      pv[e] = jj < p.dv ? zr[p.col_v + h * p.dv + jj] : ((RULE == 1 && jj == p.dv) ? 1.f : 0.f);
+      r.pv[e] = jj < p.dv ? zr[p.col_v + h * p.dv + jj] : ((RULE == 1 && jj == p.dv) ? 1.f : 0.f);
     }
     if constexpr (RULE == 1) {
-      if (sub == 0) { pi = zr[p.col_i + h] + p.b0[h]; pf = zr[p.col_f + h] + p.b0[p.H + h]; }
+      if (sub == 0) { r.pi = zr[p.col_i + h] + p.b0[h]; r.pf = zr[p.col_f + h] + p.b0[p.H + h]; }
     }
   };
   auto commit = [&](const Pre& r, int nt) {
@@ -430,6 +458,11 @@ extern "C" int dlia_state_scan(int rule, float* o, long ldo, const float* z, lon
   int CH = 12000 / per_token;
   p.CH = CH > 16 ? 16 : (CH < 1 ? 1 : CH);
   p.col_q = col_q; p.col_k = col_k; p.col_v = col_v; p.col_a = col_a; p.col_i = col_i; p.col_f = col_f; p.cap = cap; p.qscale = qscale; p.quick = quick;
+  {
+    auto al = [](const void* q) { return (uintptr_t)q % 16 == 0; };
+    const bool cols = col_q % 4 == 0 && col_k % 4 == 0 && (rule != 0 || col_a % 4 == 0) && d % 4 == 0;
+    p.vec4 = cols && ldz % 4 == 0 && al(z) && (rule != 0 || (ldw % 4 == 0 && al(wz)));
+  }
   const int ZB = (p.NC + p.CB - 1) / p.CB;
   if (ZB > dlia::kScanMaxBlocks / 2) return 2;
   p.ZB = ZB;
